@@ -225,7 +225,8 @@ class CacheManager:
                 continue
             first = min(self._first_kept_page(g, new_len), len(seq.pages[g]))
             pages = seq.pages[g]
-            for i in range(first):
+            # (a rule may keep the request's first pages for good)
+            for i in range(spec.retention.leading_pages_kept(self.page_size), first):
                 if pages[i] >= 0:
                     self.pools[g].release(pages[i])
                     seq.drop(g, i)

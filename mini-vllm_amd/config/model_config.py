@@ -706,3 +706,226 @@ class DutilixConfig(ModelConfig):
         if self.max_position_embeddings != (1 << 24):
             d["max_position_embeddings"] = self.max_position_embeddings
         return d
+
+
+# ---------------------------------------------------------------------------------------
+# Zedudra
+# ---------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class ZedudraMixer:
+    """The attention of one Zedudra layer: ``heads`` query heads on ``kv_heads`` key/value heads of size ``dim``
+    (the values are the keys, so ``vdim`` equals ``dim``), a window of ``window`` positions (the query's own among
+    them) beside the sequence's first ``keep_first``, rotation of the first ``rot_dims`` channels of a head."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int
+    keep_first: int = 0
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+
+    def to_dict(self) -> Dict[str, Any]:
+        d: Dict[str, Any] = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim,
+                             "scale": self.scale, "mask": {"size": self.window, "keep_first": self.keep_first}}
+        if self.rot_dims:
+            d["rot"] = {"dims": self.rot_dims, "base": self.rot_base}
+        return d
+
+
+@dataclass(frozen=True)
+class ZedudraFeedForward:
+    """``kind`` "dense": two projections of width ``ff`` around the xIELU activation. "moe": ``experts`` clamped gated
+    pairs of width ``ff`` (clamp at ``limit``), ``top`` used per token, chosen within ``groups_keep`` of ``groups`` groups."""
+    kind: str
+    ff: int
+    limit: float = 0.0
+    experts: int = 0
+    top: int = 0
+    groups: int = 1
+    groups_keep: int = 1
+
+    def to_dict(self) -> Dict[str, Any]:
+        if self.kind == "dense":
+            return {"kind": "dense", "ff": self.ff}
+        return {"kind": "moe", "expert": {"ff": self.ff, "limit": self.limit},
+                "router": {"experts": self.experts, "top": self.top, "groups": {"count": self.groups, "keep": self.groups_keep}}}
+
+
+@dataclass(frozen=True)
+class ZedudraLayer:
+    mixer: ZedudraMixer
+    mlp: Optional[ZedudraFeedForward] = None
+    weights_of: Optional[int] = None       # the layer whose tensors this one uses (it keeps a cache and state of its own)
+
+
+@dataclass(frozen=True)
+class ZedudraConfig(ModelConfig):
+    """Zedudra: a decoder whose ``layers`` are listed one by one. Each has a norm in groups in front of and behind
+    its attention and its feed-forward, a short causal convolution added to the attention's input (``canon.taps``),
+    softmax attention over a window and the sequence's first positions with the keys as values and a gate per head,
+    and a dense (xIELU) or routed feed-forward, or none. A layer may use another layer's tensors (``weights_of``).
+    Keys: ``vocab``, ``width``, ``layers``, ``norm.eps``, ``norm.groups``, ``canon.taps``, ``embedding.scale``."""
+
+    architecture: ClassVar[str] = "Zedudra"
+
+    vocab_size: int = 0
+    hidden_size: int = 0
+    layers: Tuple[ZedudraLayer, ...] = ()
+    norm_eps: float = 1e-6
+    norm_groups: int = 1
+    conv_taps: int = 0                     # 0: no convolution in front of the mixers
+    embedding_scale: float = 1.0
+    max_position_embeddings: int = 1 << 24
+    dtype: str = "bfloat16"
+    eos_token_ids: Tuple[int, ...] = ()
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any], where: str = "config.json") -> "ZedudraConfig":
+        raw_layers = d.get("layers")
+        if not isinstance(raw_layers, (list, tuple)) or not raw_layers:
+            raise ConfigError(f"{where}: 'layers' must be a non-empty list")
+        layers = []
+        for i, entry in enumerate(raw_layers):
+            lw = f"{where}: layers[{i}]"
+            if not isinstance(entry, dict):
+                raise ConfigError(f"{lw} must be an object")
+            if entry.get("type") != "attention":
+                raise ConfigError(f"{lw}: layer type {entry.get('type')!r} is not supported (attention)")
+            m = _section(entry, "mixer", lw)
+            mw = lw + ".mixer"
+            heads = _require(m, "heads", int, mw)
+            dim = _require(m, "dim", int, mw)
+            kv_heads, vdim, scale = m.get("kv_heads"), m.get("vdim"), m.get("scale")
+            mask = _section(m, "mask", mw)
+            rot = _section(m, "rot", mw, optional=True)
+            keep = mask.get("keep_first")
+            mixer = ZedudraMixer(
+                heads=heads, dim=dim,
+                kv_heads=heads if kv_heads is None else _typed(kv_heads, "kv_heads", int, mw),
+                vdim=dim if vdim is None else _typed(vdim, "vdim", int, mw),
+                scale=dim ** -0.5 if scale is None else _typed(scale, "scale", float, mw),
+                window=_require(mask, "size", int, mw + ".mask"),
+                keep_first=0 if keep is None else _typed(keep, "keep_first", int, mw + ".mask"),
+                rot_dims=0 if rot is None else _require(rot, "dims", int, mw + ".rot"),
+                rot_base=10000.0 if rot is None else _require(rot, "base", float, mw + ".rot"))
+            mlp = _section(entry, "mlp", lw, optional=True)
+            ff = None
+            if mlp is not None:
+                pw = lw + ".mlp"
+                mk = mlp.get("kind", "dense")
+                if mk == "dense":
+                    ff = ZedudraFeedForward(kind="dense", ff=_require(mlp, "ff", int, pw))
+                elif mk == "moe":
+                    expert = _section(mlp, "expert", pw)
+                    router = _section(mlp, "router", pw)
+                    groups = _section(router, "groups", pw + ".router", optional=True)
+                    ff = ZedudraFeedForward(
+                        kind="moe", ff=_require(expert, "ff", int, pw + ".expert"),
+                        limit=_require(expert, "limit", float, pw + ".expert"),
+                        experts=_require(router, "experts", int, pw + ".router"),
+                        top=_require(router, "top", int, pw + ".router"),
+                        groups=1 if groups is None else _require(groups, "count", int, pw + ".router.groups"),
+                        groups_keep=1 if groups is None else _require(groups, "keep", int, pw + ".router.groups"))
+                else:
+                    raise ConfigError(f"{pw}: kind {mk!r} is not supported (dense, moe)")
+            shared = entry.get("weights_of")
+            layers.append(ZedudraLayer(mixer=mixer, mlp=ff,
+                                       weights_of=None if shared is None else _typed(shared, "weights_of", int, lw)))
+        norm = _section(d, "norm", where)
+        groups = norm.get("groups")
+        canon = _section(d, "canon", where, optional=True)
+        emb = _section(d, "embedding", where, optional=True)
+        emb_scale = None if emb is None else emb.get("scale")
+        dtype = d.get("dtype", d.get("torch_dtype", "bfloat16")) or "bfloat16"
+        if str(dtype) not in _DTYPE_NAMES:
+            raise ConfigError(f"{where}: unknown dtype {dtype!r}")
+        eos = d.get("eos_token_id")
+        eos_ids: Tuple[int, ...] = ()
+        if isinstance(eos, int) and not isinstance(eos, bool):
+            eos_ids = (eos,)
+        elif isinstance(eos, (list, tuple)) and all(isinstance(e, int) for e in eos):
+            eos_ids = tuple(eos)
+        elif eos is not None:
+            raise ConfigError(f"{where}: eos_token_id must be an integer or a list of integers, got {eos!r}")
+        max_pos = d.get("max_position_embeddings")
+        cfg = cls(
+            vocab_size=_require(d, "vocab", int, where),
+            hidden_size=_require(d, "width", int, where),
+            layers=tuple(layers),
+            norm_eps=_require(norm, "eps", float, where + ".norm"),
+            norm_groups=1 if groups is None else _typed(groups, "groups", int, where + ".norm"),
+            conv_taps=0 if canon is None else _require(canon, "taps", int, where + ".canon"),
+            embedding_scale=1.0 if emb_scale is None else _typed(emb_scale, "scale", float, where + ".embedding"),
+            max_position_embeddings=(1 << 24) if max_pos is None else _typed(max_pos, "max_position_embeddings", int, where),
+            dtype=_DTYPE_NAMES[str(dtype)],
+            eos_token_ids=eos_ids,
+        )
+        cfg.validate(where)
+        return cfg
+
+    def validate(self, where: str = "config") -> None:
+        if self.vocab_size <= 0 or self.hidden_size <= 0:
+            raise ConfigError(f"{where}: vocab and width must be positive")
+        if self.norm_eps <= 0:
+            raise ConfigError(f"{where}: norm.eps must be positive, got {self.norm_eps}")
+        if self.norm_groups < 1 or self.hidden_size % self.norm_groups:
+            raise ConfigError(f"{where}: a width of {self.hidden_size} does not form {self.norm_groups} equal norm groups")
+        if self.conv_taps < 0 or self.conv_taps > 16:
+            raise ConfigError(f"{where}: canon.taps must lie in 1..16, got {self.conv_taps}")
+        for i, l in enumerate(self.layers):
+            lw = f"{where}: layers[{i}]"
+            m = l.mixer
+            if m.heads <= 0 or m.dim <= 0 or m.kv_heads <= 0 or m.heads % m.kv_heads:
+                raise ConfigError(f"{lw}: {m.heads} heads of {m.dim} are not a multiple of {m.kv_heads} kv_heads")
+            if m.vdim != m.dim:
+                raise ConfigError(f"{lw}: the values are the keys, so vdim {m.vdim} must equal dim {m.dim}")
+            if m.window < 1 or m.keep_first < 0:
+                raise ConfigError(f"{lw}: mask.size must be >= 1 and mask.keep_first >= 0")
+            if m.rot_dims < 0 or m.rot_dims % 2 or m.rot_dims > m.dim:
+                raise ConfigError(f"{lw}: rot.dims {m.rot_dims} must be even and at most dim {m.dim}")
+            if m.rot_dims and m.rot_base <= 0:
+                raise ConfigError(f"{lw}: rot.base must be positive")
+            f = l.mlp
+            if f is not None:
+                if f.ff <= 0:
+                    raise ConfigError(f"{lw}: the feed-forward width must be positive")
+                if f.kind == "moe":
+                    if f.experts < 1 or not f.limit > 0:
+                        raise ConfigError(f"{lw}: a router needs at least one expert and a positive expert.limit")
+                    if f.groups < 1 or f.experts % f.groups or not (1 <= f.groups_keep <= f.groups):
+                        raise ConfigError(f"{lw}: {f.experts} experts do not form {f.groups} equal groups of which "
+                                          f"{f.groups_keep} are kept")
+                    if not (1 <= f.top <= f.experts // f.groups * f.groups_keep):
+                        raise ConfigError(f"{lw}: top {f.top} exceeds the experts that can be chosen")
+            if l.weights_of is not None:
+                j = l.weights_of
+                if not (0 <= j < i) or self.layers[j].weights_of is not None:
+                    raise ConfigError(f"{lw}: weights_of {j} must name an earlier layer with tensors of its own")
+                if (self.layers[j].mixer, self.layers[j].mlp) != (l.mixer, l.mlp):
+                    raise ConfigError(f"{lw}: weights_of {j} names a layer with other sizes or constants than this one")
+
+    def to_dict(self) -> Dict[str, Any]:
+        layers = []
+        for l in self.layers:
+            e: Dict[str, Any] = {"type": "attention", "mixer": l.mixer.to_dict(), "mlp": None if l.mlp is None else l.mlp.to_dict()}
+            if l.weights_of is not None:
+                e["weights_of"] = l.weights_of
+            layers.append(e)
+        d: Dict[str, Any] = {
+            "architecture": self.architecture,
+            "layers": layers,
+            "norm": {"eps": self.norm_eps, "groups": self.norm_groups},
+            "embedding": {"scale": self.embedding_scale},
+            "vocab": self.vocab_size,
+            "width": self.hidden_size,
+            "torch_dtype": self.dtype,
+        }
+        if self.conv_taps:
+            d["canon"] = {"taps": self.conv_taps}
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids) if len(self.eos_token_ids) > 1 else self.eos_token_ids[0]
+        if self.max_position_embeddings != (1 << 24):
+            d["max_position_embeddings"] = self.max_position_embeddings
+        return d

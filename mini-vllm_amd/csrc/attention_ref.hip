@@ -1,11 +1,14 @@
 // Paged causal attention for any mix of query portions, one workgroup per (token, head).
 //
 // The query at absolute position p of a request sees the keys of that request at
-// positions max(0, p - window) .. p (window < 0: all of them), read from the cache pages
+// positions max(0, p - window) .. p (window < 0: all of them) and, with `first` > 0, also
+// the request's first `first` positions however far back they lie, read from the cache pages
 // through the request's block table; the step's own keys are already in the cache when
 // this runs. Scores, maximum, sum and the output accumulator are float; keys are visited
-// in tiles of 128 starting at the first visible key, so the order of additions depends
-// only on the query's position and the window, never on how the step was batched.
+// in tiles of 128 starting at the first visible key (the kept first positions in front of the
+// window's), so the order of additions depends only on the query's position, the window and
+// `first`, never on how the step was batched. With `gate`, head h's output row is multiplied by
+// sigmoid(gate[token][h]).
 //
 // Layouts:  K[page][kv_head][slot][d]   V[page][kv_head][d][slot]
 // This kernel takes every head size up to 512 and every page size; it is the float32
@@ -21,7 +24,7 @@ attention_ref_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out
                      const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                      const int* __restrict__ block_table, int bt_width, int page_size,
                      const int* __restrict__ positions, const int* __restrict__ token_seq, int H, int Hkv, int D,
-                     float scale, int window) {
+                     float scale, int window, int first, const T* __restrict__ gate, long gate_stride) {
     __shared__ float qs[AR_MAX_D];
     __shared__ float ps[AR_THREADS];
     __shared__ long voff[AR_THREADS];
@@ -38,8 +41,12 @@ attention_ref_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out
     }
     const int pos = positions[tok];
     const int kvh = head / (H / Hkv);
-    const int lo = (window >= 0 && pos - window > 0) ? pos - window : 0;
+    int lo = (window >= 0 && pos - window > 0) ? pos - window : 0;
     const int hi = pos;
+    // the kept first positions, when they all lie in front of the window, are visited first, as if
+    // they stood right in front of position lo; when they reach the window every key from 0 on is seen
+    if (first >= lo) lo = 0;
+    const int nfirst = lo > 0 ? first : 0;
     const int* bt = block_table + (size_t)seq * bt_width;
 
     const T* qrow = q + (size_t)tok * q_stride + (size_t)head * D;
@@ -51,9 +58,10 @@ attention_ref_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out
 #pragma unroll
     for (int i = 0; i < AR_MAX_D / AR_THREADS; ++i) acc[i] = 0.f;
 
-    for (int base = lo; base <= hi; base += AR_THREADS) {
-        const int j = base + tid;
-        const bool valid = j <= hi;
+    for (int base = lo - nfirst; base <= hi; base += AR_THREADS) {
+        const int jj0 = base + tid;
+        const int j = jj0 < lo ? jj0 - (lo - nfirst) : jj0;
+        const bool valid = jj0 <= hi;
         float s = -INFINITY;
         long vo = 0;
         if (valid) {
@@ -87,7 +95,8 @@ attention_ref_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out
         }
         __syncthreads();
     }
-    const float inv = 1.f / l;
+    float inv = 1.f / l;
+    if (gate != nullptr) inv *= 1.f / (1.f + expf(-to_f(gate[(size_t)tok * gate_stride + head])));
 #pragma unroll
     for (int i = 0; i < AR_MAX_D / AR_THREADS; ++i) {
         const int d = tid + i * AR_THREADS;
@@ -98,7 +107,8 @@ attention_ref_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out
 extern "C" int mv_attention_ref(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
                                 const void* v_pages, const int* block_table, int bt_width, int page_size,
                                 const int* positions, const int* token_seq, int n, int H, int Hkv, int D,
-                                float scale, int window, int dtype, hipStream_t stream) {
+                                float scale, int window, int first, const void* gate, long gate_stride, int dtype,
+                                hipStream_t stream) {
     MV_REQUIRE(n >= 0 && H > 0 && Hkv > 0 && D > 0, "attention: bad sizes n=%d H=%d Hkv=%d D=%d", n, H, Hkv, D);
     MV_REQUIRE(H % Hkv == 0, "attention: %d query heads are not a multiple of %d key/value heads", H, Hkv);
     MV_REQUIRE(D <= AR_MAX_D, "attention: head_dim %d exceeds the supported maximum %d", D, AR_MAX_D);
@@ -106,11 +116,12 @@ extern "C" int mv_attention_ref(const void* q, long q_stride, void* out, long ou
                bt_width);
     MV_REQUIRE(q_stride >= (long)H * D && out_stride >= (long)H * D, "attention: row strides too small");
     MV_REQUIRE(H <= 65535, "attention: too many heads %d", H);
+    MV_REQUIRE(first >= 0 && (gate == nullptr || gate_stride >= H), "attention: bad count of kept first positions or gate rows too short");
     if (n == 0) return 0;
     MV_DISPATCH_T(dtype, "attention",
                   hipLaunchKernelGGL(attention_ref_kernel<T>, dim3(n, H), dim3(AR_THREADS), 0, stream, (const T*)q,
                                      q_stride, (T*)out, out_stride, (const T*)k_pages, (const T*)v_pages,
                                      block_table, bt_width, page_size, positions, token_seq, H, Hkv, D, scale,
-                                     window));
+                                     window, first, (const T*)gate, gate_stride));
     return mv_check_launch("attention");
 }

@@ -891,6 +891,32 @@ extern "C" int mv_swiglu(const void* gate_up, void* out, int n, int I, int dtype
 }
 
 // ---------------------------------------------------------------------------------------
+// xIELU, element by element, with its two positive constants a_pos and a_neg:
+//   z > 0 : a_pos z^2 + z / 2        z <= 0 : a_neg (exp(z) - 1 - z) + z / 2
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void xielu_kernel(const T* __restrict__ x, long ldx, T* __restrict__ out, long ldo, int cols, long total,
+                             float a_pos, float a_neg) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const long r = i / cols, c = i % cols;
+    const float z = to_f(x[r * ldx + c]);
+    const float v = z > 0.f ? fmaf(a_pos * z, z, 0.5f * z) : fmaf(a_neg, expm1f(z) - z, 0.5f * z);
+    out[r * ldo + c] = from_f<T>(v);
+}
+
+extern "C" int mv_xielu(const void* x, long ldx, void* out, long ldo, int n, int cols, float a_pos, float a_neg, int dtype,
+                        hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && cols > 0 && ldx >= cols && ldo >= cols && x && out, "xielu: bad sizes n=%d cols=%d", n, cols);
+    const long total = (long)n * cols;
+    if (total == 0) return 0;
+    MV_DISPATCH_T(dtype, "xielu",
+                  hipLaunchKernelGGL(xielu_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (const T*)x,
+                                     ldx, (T*)out, ldo, cols, total, a_pos, a_neg));
+    return mv_check_launch("xielu");
+}
+
+// ---------------------------------------------------------------------------------------
 // A norm behind a sublayer, the residual add, and the norm in front of the next sublayer:
 //   v = resid[r] + y[r] / sqrt(mean(y[r]^2) + eps_a) * wa ;  resid[r] = v ;
 //   out[r] = v / sqrt(mean(v^2) + eps_b) * wb                          (out == null: the add alone)

@@ -7,13 +7,22 @@
 //                      a chosen expert is its score divided by the chosen scores' sum (+ sum_eps).
 //                      Leaves the weights dense, [n][E] with zeros for the others, and as lists
 //                      (ids [n][top], weights [n][top], in the order chosen).
+//                      Options (`flags`): MR_SIGMOID scores = sigmoid(logit) instead of the softmax;
+//                      MR_WORTH_TOP2 a group's worth is the sum of its two largest choices (of its one
+//                      choice when it has one); MR_RAW_WEIGHTS the weights are the chosen scores as they
+//                      are, not divided by their sum.
 //   moe_swiglu_scale   act[t][e][c] = weight[t][e] * silu(gate[t][e][c]) * up[t][e][c]: the gated pair of
 //                      every expert with the router's weight applied before the one rounding, so that
-//                      one product with all experts' down matrices side by side sums the chosen experts
+//                      one product with all experts' down matrices side by side sums the chosen experts.
+//                      With a `limit` > 0 the pair is the clamped one: g = min(gate, limit),
+//                      u = clamp(up, -limit, limit), act = weight * g * sigmoid(slope * g) * (u + 1).
 //   moe_identity_add   y[t] += (sum of the weights of the identity experts of t) * h[t]
 #include "dispatch.h"
 
 #define MR_MAX_E 1024
+#define MR_SIGMOID 1
+#define MR_WORTH_TOP2 2
+#define MR_RAW_WEIGHTS 4
 
 // the largest value over the wave and the smallest index that holds it (index INT_MAX: nothing left)
 __device__ __forceinline__ void wave_argmax(float& best, int& at) {
@@ -29,24 +38,29 @@ __device__ __forceinline__ void wave_argmax(float& best, int& at) {
 
 __global__ void __launch_bounds__(64)
 moe_route_kernel(const float* __restrict__ logits, long ld, int E, WeightPtr correction, int has_correction, int groups, int keep,
-                 int top, float sum_eps, float* __restrict__ dense, int* __restrict__ ids, float* __restrict__ weights) {
+                 int top, float sum_eps, int flags, float* __restrict__ dense, int* __restrict__ ids, float* __restrict__ weights) {
     __shared__ float score[MR_MAX_E];
     __shared__ float choice[MR_MAX_E];
     __shared__ float worth[MR_MAX_E];          // of the groups
     __shared__ int open_group[MR_MAX_E];       // 1: its experts may be chosen
     const int t = blockIdx.x, lane = threadIdx.x;
     const float* z = logits + (size_t)t * ld;
-    float mx = -INFINITY;
-    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
-    mx = wave_max(mx);
-    float sum = 0.f;
-    for (int e = lane; e < E; e += 64) {
-        const float p = expf(z[e] - mx);
-        score[e] = p;
-        sum += p;
+    float inv = 1.f;
+    if (flags & MR_SIGMOID) {
+        for (int e = lane; e < E; e += 64) score[e] = 1.f / (1.f + expf(-z[e]));
+    } else {
+        float mx = -INFINITY;
+        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int e = lane; e < E; e += 64) {
+            const float p = expf(z[e] - mx);
+            score[e] = p;
+            sum += p;
+        }
+        sum = wave_sum(sum);
+        inv = 1.f / sum;
     }
-    sum = wave_sum(sum);
-    const float inv = 1.f / sum;
     for (int e = lane; e < E; e += 64) {
         const float s = score[e] * inv;
         score[e] = s;
@@ -56,9 +70,17 @@ moe_route_kernel(const float* __restrict__ logits, long ld, int E, WeightPtr cor
     __syncthreads();
     const int per = E / groups;
     for (int g = lane; g < groups; g += 64) {
-        float w = -INFINITY;
-        for (int i = 0; i < per; ++i) w = fmaxf(w, choice[g * per + i]);
-        worth[g] = w;
+        float w = -INFINITY, second = -INFINITY;
+        for (int i = 0; i < per; ++i) {
+            const float c = choice[g * per + i];
+            if (c > w) {
+                second = w;
+                w = c;
+            } else if (c > second) {
+                second = c;
+            }
+        }
+        worth[g] = ((flags & MR_WORTH_TOP2) && per > 1) ? w + second : w;
         open_group[g] = keep >= groups ? 1 : 0;
     }
     __syncthreads();
@@ -102,7 +124,7 @@ moe_route_kernel(const float* __restrict__ logits, long ld, int E, WeightPtr cor
         __syncthreads();
     }
     if (lane < top) {
-        const float w = my_id >= 0 ? my_w / (picked_sum + sum_eps) : 0.f;
+        const float w = my_id >= 0 ? ((flags & MR_RAW_WEIGHTS) ? my_w : my_w / (picked_sum + sum_eps)) : 0.f;
         ids[(size_t)t * top + lane] = my_id;
         weights[(size_t)t * top + lane] = w;
         if (my_id >= 0) dense[(size_t)t * E + my_id] = w;
@@ -110,7 +132,7 @@ moe_route_kernel(const float* __restrict__ logits, long ld, int E, WeightPtr cor
 }
 
 extern "C" int mv_moe_route(const float* logits, long ld, int n, int E, const void* correction, int weight_dtype, int groups,
-                            int keep, int top, float sum_eps, float* dense, int* ids, float* weights, hipStream_t stream) {
+                            int keep, int top, float sum_eps, int flags, float* dense, int* ids, float* weights, hipStream_t stream) {
     MV_REQUIRE(n >= 0 && E > 0 && E <= MR_MAX_E && ld >= E, "moe_route: bad sizes n=%d E=%d (at most %d)", n, E, MR_MAX_E);
     MV_REQUIRE(groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups, "moe_route: %d groups of which %d stay do not fit %d experts",
                groups, keep, E);
@@ -119,7 +141,7 @@ extern "C" int mv_moe_route(const float* logits, long ld, int n, int E, const vo
     if (n == 0) return 0;
     WeightPtr c{correction, weight_dtype};
     hipLaunchKernelGGL(moe_route_kernel, dim3(n), dim3(64), 0, stream, logits, ld, E, c, correction ? 1 : 0, groups, keep, top,
-                       sum_eps, dense, ids, weights);
+                       sum_eps, flags, dense, ids, weights);
     return mv_check_launch("moe_route");
 }
 
@@ -127,7 +149,7 @@ extern "C" int mv_moe_route(const float* logits, long ld, int n, int E, const vo
 template <typename T>
 __global__ void __launch_bounds__(256)
 moe_swiglu_scale_kernel(const T* __restrict__ gate_up, long ld, const float* __restrict__ dense, int ld_dense, int E, int F,
-                        T* __restrict__ act, long total) {
+                        T* __restrict__ act, long total, float limit, float slope) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const long EF = (long)E * F;
@@ -136,20 +158,25 @@ moe_swiglu_scale_kernel(const T* __restrict__ gate_up, long ld, const float* __r
     float v = 0.f;
     if (w != 0.f) {
         const float g = to_f(gate_up[t * ld + c]), u = to_f(gate_up[t * ld + EF + c]);
-        v = w * (g / (1.f + expf(-g))) * u;
+        if (limit > 0.f) {
+            const float gc = fminf(g, limit), uc = fminf(fmaxf(u, -limit), limit);
+            v = w * (gc / (1.f + expf(-slope * gc))) * (uc + 1.f);
+        } else {
+            v = w * (g / (1.f + expf(-g))) * u;
+        }
     }
     act[t * EF + c] = from_f<T>(v);
 }
 
 extern "C" int mv_moe_swiglu_scale(const void* gate_up, long ld, const float* dense, int ld_dense, int n, int E, int F, void* act,
-                                   int dtype, hipStream_t stream) {
+                                   float limit, float slope, int dtype, hipStream_t stream) {
     MV_REQUIRE(n >= 0 && E > 0 && F > 0 && ld >= 2L * E * F && ld_dense >= E, "moe_swiglu_scale: bad sizes n=%d E=%d F=%d", n, E, F);
     MV_REQUIRE(gate_up && dense && act, "moe_swiglu_scale: missing operand");
     const long total = (long)n * E * F;
     if (total == 0) return 0;
     MV_DISPATCH_T(dtype, "moe_swiglu_scale",
                   hipLaunchKernelGGL(moe_swiglu_scale_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
-                                     (const T*)gate_up, ld, dense, ld_dense, E, F, (T*)act, total));
+                                     (const T*)gate_up, ld, dense, ld_dense, E, F, (T*)act, total, limit, slope));
     return mv_check_launch("moe_swiglu_scale");
 }
 

@@ -744,6 +744,61 @@ conv_state_kernel(const T* __restrict__ packed, long ld, int C, int taps, T* __r
     for (int i = 0; i < taps - 1; ++i) hist[(size_t)i * C + c] = keep[i];
 }
 
+// A causal convolution over time added to its own input, channel by channel:
+//   out[t][c] = h[t][c] + sum_j w[c][j] * h[t - taps + 1 + j][c]      (the last tap multiplies h[t] itself)
+// Rows in front of a request's first row of the step come from its kept inputs conv_state[slot][taps-1][C]
+// (zeros at a request's start); conv_state_kernel moves them on afterwards. The sum starts from h[t] and takes
+// the taps in order, so a row's value does not depend on where the step cut the request.
+template <typename T>
+__global__ void __launch_bounds__(256)
+input_conv_kernel(const T* __restrict__ h, long ldh, T* __restrict__ out, long ldo, WeightPtr w, int taps,
+                  const T* __restrict__ conv_state, const int* __restrict__ token_seq, const int* __restrict__ cu_seqlens,
+                  const int* __restrict__ state_slots, int C) {
+    const int t = blockIdx.x;
+    const int seq = token_seq[t];
+    T* o = out + (size_t)t * ldo;
+    if (seq < 0) {
+        for (int c = threadIdx.x; c < C; c += blockDim.x) o[c] = from_f<T>(0.f);
+        return;
+    }
+    const int first = cu_seqlens[seq];
+    const T* hist = taps > 1 ? conv_state + (size_t)state_slots[seq] * (taps - 1) * C : nullptr;
+    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+        float acc = to_f(h[(size_t)t * ldh + c]);
+        for (int j = 0; j < taps; ++j) {
+            const int r = t - (taps - 1) + j;
+            const float x = r >= first ? to_f(h[(size_t)r * ldh + c]) : to_f(hist[(size_t)(taps - 1 + (r - first)) * C + c]);
+            acc = fmaf(w.at((size_t)c * taps + j), x, acc);
+        }
+        o[c] = from_f<T>(acc);
+    }
+}
+
+// h, ldh, out, ldo: [n][C] rows; w [C][taps]; conv_state [slots][taps-1][C] in the activation type (may be null with one tap)
+extern "C" int mv_input_conv(const void* h, long ldh, void* out, long ldo, const void* w, int weight_dtype, int taps,
+                             void* conv_state, const int* token_seq, const int* cu_seqlens, const int* state_slots, int n,
+                             int n_seqs, int C, int dtype, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && n_seqs >= 0 && C > 0 && ldh >= C && ldo >= C, "input_conv: bad sizes n=%d C=%d", n, C);
+    MV_REQUIRE(taps >= 1 && taps <= MS_MAX_TAPS, "input_conv: %d taps, 1 to %d are served", taps, MS_MAX_TAPS);
+    MV_REQUIRE(h != out, "input_conv: a row reads the rows in front of it, the output must be another buffer");
+    MV_REQUIRE(mv_valid_dtype(weight_dtype) && h && out && w && (conv_state || taps == 1) && token_seq && cu_seqlens && state_slots,
+               "input_conv: missing operand");
+    MV_REQUIRE((C + 255) / 256 <= 65535, "input_conv: too many channels");
+    if (n == 0) return 0;
+    WeightPtr wp{w, weight_dtype};
+    MV_DISPATCH_T(dtype, "input_conv",
+                  hipLaunchKernelGGL(input_conv_kernel<T>, dim3(n), dim3(256), 0, stream, (const T*)h, ldh, (T*)out, ldo, wp, taps,
+                                     (const T*)conv_state, token_seq, cu_seqlens, state_slots, C));
+    if (mv_check_launch("input_conv")) return 1;
+    if (taps > 1 && n_seqs > 0) {
+        MV_DISPATCH_T(dtype, "conv_state",
+                      hipLaunchKernelGGL(conv_state_kernel<T>, dim3(n_seqs, (unsigned)((C + 255) / 256)), dim3(256), 0, stream,
+                                         (const T*)h, ldh, C, taps, (T*)conv_state, cu_seqlens, state_slots));
+        return mv_check_launch("conv_state");
+    }
+    return 0;
+}
+
 extern "C" int mv_gdelta_prepare(const void* packed, long ld, int n, int n_seqs, int H, int G, int DK, int DV, int taps,
                                  const void* conv_w, const void* a_log, const void* dt_bias, int weight_dtype,
                                  void* conv_state, float unit_eps, const int* token_seq, const int* cu_seqlens,

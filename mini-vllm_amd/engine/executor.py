@@ -415,7 +415,8 @@ class Executor:
             spec = self.groups[g]
             first_page = spec.retention.first_kept_pages(starts, self.page_size)
             idx = np.arange(w, dtype=np.int64)[None, :]
-            touched = (idx >= first_page[:, None]) & (idx <= last_page[:, None])
+            touched = ((idx >= first_page[:, None]) | (idx < spec.retention.leading_pages_kept(self.page_size))) \
+                & (idx <= last_page[:, None])
             ids = bt[:S][touched]
             if check_pages and ids.size and (ids.min() < 0 or ids.max() >= self.group_pages[g]):
                 raise ValueError(f"cache group {g}: a block table names a page outside the pool of "

@@ -43,8 +43,24 @@ _SIGNATURES = {
     "mv_swiglu": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "mv_gemm_ref": (c_int, [c_void_p, c_long, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_int,
                             c_int, c_int, c_int, c_void_p]),
+    # q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width, page_size, positions, token_seq, n, H, Hkv, D,
+    # scale, window, first, gate, gate_stride, dtype, stream
     "mv_attention_ref": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                                 c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p]),
+                                 c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_long,
+                                 c_int, c_void_p]),
+    # resid, x, ldx, delta, weight, weight_dtype, eps, groups, out, ldo, rows, n_out, h, dtype, stream
+    "mv_group_norm_rows": (c_int, [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_long,
+                                   c_void_p, c_int, c_int, c_int, c_void_p]),
+    # y, ldy, wa, wa_dtype, eps_a, resid, wb, wb_dtype, eps_b, groups, out, n, h, conv_taps, conv_w, conv_w_dtype, conv_state,
+    # token_seq, state_slots, dtype, stream
+    "mv_group_norm_add_norm": (c_int, [c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_float, c_int,
+                                       c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                       c_void_p]),
+    # h, ldh, out, ldo, w, weight_dtype, taps, conv_state, token_seq, cu_seqlens, state_slots, n, n_seqs, C, dtype, stream
+    "mv_input_conv": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                              c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    # x, ldx, out, ldo, n, cols, a_pos, a_neg, dtype, stream
+    "mv_xielu": (c_int, [c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_float, c_float, c_int, c_void_p]),
     # h, ldh, out, ldo, mix, mix_dtype, state, token_seq, cu_seqlens, state_slots, n, width, dtype, stream
     "mv_token_shift": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_int, c_int, c_int, c_void_p]),
@@ -192,11 +208,12 @@ _OPTIONAL_SIGNATURES = {
     "mv_attention_latent_split": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                           c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_long, c_int,
                                           c_void_p]),
-    # logits, ld, n, E, correction, weight_dtype, groups, keep, top, sum_eps, dense, ids, weights, stream
-    "mv_moe_route": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p,
-                             c_void_p, c_void_p]),
-    # gate_up, ld, dense, ld_dense, n, E, F, act, dtype, stream
-    "mv_moe_swiglu_scale": (c_int, [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p]),
+    # logits, ld, n, E, correction, weight_dtype, groups, keep, top, sum_eps, flags, dense, ids, weights, stream
+    "mv_moe_route": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p,
+                             c_void_p, c_void_p, c_void_p]),
+    # gate_up, ld, dense, ld_dense, n, E, F, act, limit, slope, dtype, stream
+    "mv_moe_swiglu_scale": (c_int, [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_float, c_float, c_int,
+                                    c_void_p]),
     # y, ldy, h, ldh, dense, ld_dense, first, count, n, width, set, dtype, stream
     "mv_moe_identity_add": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_void_p]),

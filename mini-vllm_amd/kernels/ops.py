@@ -374,18 +374,25 @@ class Ops:
                            rope_table: Optional[torch.Tensor], interleaved: bool,
                            k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor],
                            block_table: Optional[torch.Tensor], page_size: int,
-                           unit_offset: bool = False, value_dim: Optional[int] = None) -> None:
+                           unit_offset: bool = False, value_dim: Optional[int] = None, value_from_key: bool = False,
+                           extra_columns: int = 0) -> None:
         """In place on the rows of ``qkv`` = [q | k | v]: per-head RMSNorm of q and k (when
         weights are given), rotary embedding (when a table is given); k and v are written to
         the cache pages when pages are given. Without pages the rows hold only q. With
         ``value_dim`` a value row has that size instead of ``head_dim``, and the rows may hold
-        further columns behind v (nothing touches them)."""
+        further columns behind v (nothing touches them). With ``value_from_key`` the rows are
+        [q | k] and the value pages take the keys as the rows hold them, before norm and rotation
+        (the key columns themselves are never rewritten: rotated keys go to the key pages only).
+        ``extra_columns``: columns behind these that nothing touches."""
         self._act(qkv, "qkv")
         n = qkv.shape[0]
         store = k_pages is not None
         vdim = head_dim if value_dim is None else int(value_dim)
-        width = num_heads * head_dim + (num_kv_heads * (head_dim + vdim) if store else 0)
-        if qkv.dim() != 2 or qkv.stride(1) != 1 or (qkv.shape[1] != width if value_dim is None else qkv.shape[1] < width):
+        if value_from_key and (vdim != head_dim or not store):
+            raise KernelLibraryError("qk_norm_rope_store: values taken from the keys have the keys' size and go to pages")
+        width = num_heads * head_dim + (num_kv_heads * (head_dim + (0 if value_from_key else vdim)) if store else 0)
+        if qkv.dim() != 2 or qkv.stride(1) != 1 or (qkv.shape[1] != width + extra_columns if value_dim is None and not extra_columns
+                                                    else qkv.shape[1] < width + extra_columns):
             raise KernelLibraryError(f"qk_norm_rope_store: qkv {tuple(qkv.shape)} does not hold {width} columns")
         for t, what in ((positions, "positions"), (token_seq, "token_seq")):
             _dev(t, what)
@@ -437,7 +444,7 @@ class Ops:
         self._note("mv_qk_norm_rope_store", n * (width + q_dim + (2 * kv_dim if store else 0)) * qkv.element_size()
                    + (n * rot * 4 if rope_table is not None else 0), 10 * n * (q_dim + (kv_dim if store else 0)))
         self.lib.call("mv_qk_norm_rope_store", qkv.data_ptr(), stride, 0, q_dim,
-                      q_dim + kv_dim, positions.data_ptr(), token_seq.data_ptr(), _ptr(block_table), bt_width,
+                      q_dim if value_from_key else q_dim + kv_dim, positions.data_ptr(), token_seq.data_ptr(), _ptr(block_table), bt_width,
                       page_size, _ptr(k_pages), _ptr(v_pages), n, num_heads, num_kv_heads, head_dim,
                       _ptr(q_weight), _ptr(k_weight), wcode, float(eps), int(unit_offset), _ptr(rope_table), rot,
                       int(interleaved), mode, self.code, self._stream())
@@ -467,6 +474,123 @@ class Ops:
         self.lib.call("mv_token_shift", h.data_ptr(), h.stride(0) if n > 1 else w, out.data_ptr(),
                       out.stride(0) if n > 1 else w, mix.data_ptr(), _weight_code(mix, "shift weight"), state.data_ptr(),
                       token_seq.data_ptr(), cu_seqlens.data_ptr(), state_slots.data_ptr(), n, w, self.code, self._stream())
+
+    def input_conv(self, h: torch.Tensor, taps: torch.Tensor, state: Optional[torch.Tensor], token_seq: torch.Tensor,
+                   cu_seqlens: torch.Tensor, state_slots: torch.Tensor, n_seqs: int, out: torch.Tensor) -> None:
+        """out[t] = h[t] + sum_j taps[:, j] * h[t - T + 1 + j] along each request's rows (T = taps.shape[1], the last tap
+        multiplies h[t]); the rows in front of a request's first row of the step are state[slot] [T - 1, w], which then
+        takes the request's last T - 1 rows. h, out [n, w]; taps [w, T]; state [slots, T - 1, w] (None with one tap)."""
+        self._act(h, "convolution input"); self._act(out, "convolution output"); _dev(taps, "convolution taps")
+        n, w = h.shape
+        if out.shape != h.shape or h.stride(1) != 1 or out.stride(1) != 1 or out.data_ptr() == h.data_ptr():
+            raise KernelLibraryError("input_conv: input and output must be two [n, w] buffers")
+        if taps.dim() != 2 or taps.shape[0] != w or not taps.is_contiguous():
+            raise KernelLibraryError(f"input_conv: taps {tuple(taps.shape)} do not fit rows of {w}")
+        T = taps.shape[1]
+        if T > 1:
+            self._act(state, "convolution state")
+            if tuple(state.shape[1:]) != (T - 1, w) or not state.is_contiguous():
+                raise KernelLibraryError(f"input_conv: state {tuple(state.shape)} does not hold {T - 1} rows of {w}")
+        self._ints(n, token_seq=(token_seq, n), cu_seqlens=(cu_seqlens, n_seqs + 1), state_slots=(state_slots, n_seqs))
+        self._note("mv_input_conv", self._size(h, out) + (T - 1) * n_seqs * w * h.element_size() * 2, 2 * T * n * w)
+        self.lib.call("mv_input_conv", h.data_ptr(), h.stride(0) if n > 1 else w, out.data_ptr(), out.stride(0) if n > 1 else w,
+                      taps.data_ptr(), _weight_code(taps, "convolution taps"), T, _ptr(state) if T > 1 else 0,
+                      token_seq.data_ptr(), cu_seqlens.data_ptr(), state_slots.data_ptr(), n, n_seqs, w, self.code, self._stream())
+
+    def group_norm(self, weight: torch.Tensor, eps: float, groups: int, out: torch.Tensor, resid: Optional[torch.Tensor] = None,
+                   x: Optional[torch.Tensor] = None, delta: Optional[torch.Tensor] = None,
+                   rows: Optional[torch.Tensor] = None) -> None:
+        """RMS norm in ``groups`` equal runs of neighbouring columns, times ``weight``. Either of the float32 residual
+        ``resid`` [n, h] (plus ``delta``; without ``rows`` the sum goes back to ``resid``; with ``rows`` int32 only those rows
+        are normalised and nothing is written back) or of the activation rows ``x`` [n, h]."""
+        if (resid is None) == (x is None):
+            raise KernelLibraryError("group_norm: either the residual or activation rows")
+        src = resid if resid is not None else x
+        _dev(src, "norm input"); self._act(out, "norm output"); _dev(weight, "norm weight")
+        n, h = src.shape
+        if resid is not None and (resid.dtype != torch.float32 or not resid.is_contiguous()):
+            raise KernelLibraryError("group_norm: the residual must be a contiguous float32 [n, h]")
+        if x is not None:
+            self._act(x, "norm input")
+            if x.dim() != 2 or x.stride(1) != 1 or delta is not None or rows is not None:
+                raise KernelLibraryError("group_norm: activation rows are normalised as they are")
+        if delta is not None:
+            self._act(delta, "delta")
+            if delta.shape != src.shape or not delta.is_contiguous():
+                raise KernelLibraryError(f"group_norm: delta {tuple(delta.shape)} does not match {tuple(src.shape)}")
+        n_out = n
+        if rows is not None:
+            _dev(rows, "rows")
+            if rows.dtype != torch.int32:
+                raise KernelLibraryError("group_norm: rows must be int32")
+            n_out = rows.numel()
+        if weight.numel() != h or not weight.is_contiguous() or groups < 1 or h % groups:
+            raise KernelLibraryError(f"group_norm: weight of {weight.numel()} elements / {groups} groups for rows of {h}")
+        if out.dim() != 2 or out.shape[0] < n_out or out.shape[1] != h or out.stride(1) != 1:
+            raise KernelLibraryError(f"group_norm: output {tuple(out.shape)} does not fit [{n_out}, {h}]")
+        self._note("mv_group_norm_rows", n_out * h * (src.element_size() * (2 if resid is not None and delta is not None and rows is None else 1)
+                                                      + (delta.element_size() if delta is not None else 0) + out.element_size()),
+                   4 * n_out * h)
+        self.lib.call("mv_group_norm_rows", _ptr(resid), _ptr(x), (x.stride(0) if n > 1 else h) if x is not None else 0,
+                      _ptr(delta), weight.data_ptr(), _weight_code(weight, "norm weight"), float(eps), int(groups),
+                      out.data_ptr(), out.stride(0) if out.shape[0] > 1 else h, _ptr(rows), n_out, h, self.code, self._stream())
+
+    def group_norm_add_norm(self, y: torch.Tensor, norm_y, resid: torch.Tensor, norm_next, out: Optional[torch.Tensor],
+                            groups: int, conv: Optional[tuple] = None) -> None:
+        """resid += gnorm(y) * w (``norm_y`` = (weight, eps)); with ``norm_next`` of the same form, out = gnorm(resid) * w'.
+        Both norms work in ``groups`` runs of columns; the sum stays float32 in between.
+
+        ``conv`` = (taps [h, T], state [slots, T - 1, h] or None, token_seq, state_slots), for steps in which every request
+        brings one token: ``out`` gets the rows after the input convolution that ``input_conv`` would apply to them."""
+        self._act(y, "sublayer output"); _dev(resid, "residual")
+        n, h = resid.shape
+        if resid.dtype != torch.float32 or not resid.is_contiguous() or tuple(y.shape) != (n, h) or y.stride(1) != 1:
+            raise KernelLibraryError("group_norm_add_norm: a float32 residual [n, h] and an output of the same shape are needed")
+        wa, eps_a = norm_y
+        _dev(wa, "norm weight")
+        if wa.numel() != h or not wa.is_contiguous() or groups < 1 or h % groups:
+            raise KernelLibraryError(f"group_norm_add_norm: weight of {wa.numel()} elements / {groups} groups for rows of {h}")
+        wb, eps_b, wb_code = None, 1.0, DTYPE_F32
+        if out is not None:
+            if norm_next is None:
+                raise KernelLibraryError("group_norm_add_norm: an output needs the second norm")
+            self._act(out, "norm output")
+            wb, eps_b = norm_next
+            _dev(wb, "norm weight")
+            wb_code = _weight_code(wb, "norm weight")
+            if wb.numel() != h or not wb.is_contiguous() or tuple(out.shape) != (n, h) or not out.is_contiguous():
+                raise KernelLibraryError("group_norm_add_norm: the second norm's weight or output does not fit")
+        taps = state = tsq = slots = None
+        T, taps_code = 0, DTYPE_F32
+        if conv is not None:
+            taps, state, tsq, slots = conv
+            if out is None:
+                raise KernelLibraryError("group_norm_add_norm: a convolution needs the second norm and its output")
+            _dev(taps, "convolution taps")
+            taps_code = _weight_code(taps, "convolution taps")
+            if taps.dim() != 2 or taps.shape[0] != h or not taps.is_contiguous():
+                raise KernelLibraryError(f"group_norm_add_norm: taps {tuple(taps.shape)} do not fit rows of {h}")
+            T = taps.shape[1]
+            if T > 1:
+                self._act(state, "convolution state")
+                if tuple(state.shape[1:]) != (T - 1, h) or not state.is_contiguous():
+                    raise KernelLibraryError(f"group_norm_add_norm: state {tuple(state.shape)} does not hold {T - 1} rows of {h}")
+            self._ints(n, token_seq=(tsq, n), state_slots=(slots, 1))
+        self._note("mv_group_norm_add_norm", self._size(y, out) + 2 * self._size(resid), 8 * n * h)
+        self.lib.call("mv_group_norm_add_norm", y.data_ptr(), y.stride(0) if n > 1 else h, wa.data_ptr(),
+                      _weight_code(wa, "norm weight"), float(eps_a), resid.data_ptr(), _ptr(wb), wb_code, float(eps_b), int(groups),
+                      _ptr(out), n, h, T, _ptr(taps), taps_code, _ptr(state) if T > 1 else 0, _ptr(tsq), _ptr(slots),
+                      self.code, self._stream())
+
+    def xielu(self, x: torch.Tensor, a_pos: float, a_neg: float, out: torch.Tensor) -> None:
+        """out = a_pos x^2 + x / 2 where x > 0, a_neg (exp(x) - 1 - x) + x / 2 elsewhere; x, out [n, cols] (may be the same)."""
+        self._act(x, "activation input"); self._act(out, "activation output")
+        if x.dim() != 2 or out.shape != x.shape or x.stride(1) != 1 or out.stride(1) != 1:
+            raise KernelLibraryError("xielu: input and output must be [n, cols] with a contiguous last dimension")
+        n, cols = x.shape
+        self._note("mv_xielu", self._size(x, out), 6 * n * cols)
+        self.lib.call("mv_xielu", x.data_ptr(), x.stride(0) if n > 1 else cols, out.data_ptr(), out.stride(0) if n > 1 else cols,
+                      n, cols, float(a_pos), float(a_neg), self.code, self._stream())
 
     def _delta_weights(self, heads: int, dim: int, rank: int, w2t: torch.Tensor, w0: torch.Tensor, a_bias: torch.Tensor,
                        what: str) -> int:
@@ -882,11 +1006,17 @@ class Ops:
     # ------------------------------------------------------------------------------------
     # mixture of experts
     def moe_route(self, logits: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int, top: int,
-                  sum_eps: float, dense: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -> None:
+                  sum_eps: float, dense: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, scoring: str = "softmax",
+                  group_worth: str = "max", normalize: bool = True) -> None:
         """From float32 router logits [n, E]: scores = softmax over E; the ``top`` largest of scores + correction among the
         experts of the ``keep`` groups (of ``groups`` equal runs of neighbours) whose largest such number is largest are
         chosen; a chosen expert's weight is its score / (sum of the chosen scores + sum_eps). dense float32 [n, E] gets the
-        weights (zero elsewhere), ids int32 / weights float32 [n, top] the chosen experts in the order of choice."""
+        weights (zero elsewhere), ids int32 / weights float32 [n, top] the chosen experts in the order of choice.
+        ``scoring`` "sigmoid": scores = sigmoid(logit); ``group_worth`` "top2": a group is worth the sum of its two
+        largest numbers; ``normalize`` False: the weights are the chosen scores themselves."""
+        if scoring not in ("softmax", "sigmoid") or group_worth not in ("max", "top2"):
+            raise KernelLibraryError(f"moe_route: unknown scoring {scoring!r} or group worth {group_worth!r}")
+        flags = (1 if scoring == "sigmoid" else 0) | (2 if group_worth == "top2" else 0) | (0 if normalize else 4)
         _dev(logits, "router logits")
         n, E = logits.shape
         if logits.dtype != torch.float32 or logits.stride(1) != 1:
@@ -903,11 +1033,13 @@ class Ops:
         self._note("mv_moe_route", self._size(logits, dense, ids, weights), 20 * n * E)
         self.lib.call("mv_moe_route", logits.data_ptr(), logits.stride(0) if n > 1 else E, n, E, _ptr(correction),
                       _weight_code(correction, "router correction") if correction is not None else DTYPE_F32, groups, keep,
-                      top, float(sum_eps), dense.data_ptr(), ids.data_ptr(), weights.data_ptr(), self._stream())
+                      top, float(sum_eps), flags, dense.data_ptr(), ids.data_ptr(), weights.data_ptr(), self._stream())
 
-    def moe_swiglu_scale(self, gate_up: torch.Tensor, dense: torch.Tensor, experts: int, ff: int, out: torch.Tensor) -> None:
+    def moe_swiglu_scale(self, gate_up: torch.Tensor, dense: torch.Tensor, experts: int, ff: int, out: torch.Tensor,
+                         limit: float = 0.0, slope: float = 1.0) -> None:
         """out[t, e, c] = dense[t, e] * silu(gate_up[t, e*ff + c]) * gate_up[t, experts*ff + e*ff + c] (zero where the
-        weight is zero, whatever the products hold)."""
+        weight is zero, whatever the products hold). With ``limit`` > 0 the clamped pair instead: g = min(gate, limit),
+        u = clamp(up, -limit, limit), out = dense * g * sigmoid(slope * g) * (u + 1)."""
         self._act(gate_up, "gate_up"); self._act(out, "expert activations"); _dev(dense, "dense weights")
         n = gate_up.shape[0]
         if tuple(gate_up.shape) != (n, 2 * experts * ff) or gate_up.stride(1) != 1 or tuple(out.shape) != (n, experts * ff) \
@@ -916,7 +1048,8 @@ class Ops:
             raise KernelLibraryError("moe_swiglu_scale: operands do not fit")
         self._note("mv_moe_swiglu_scale", self._size(gate_up, out), 8 * out.numel())
         self.lib.call("mv_moe_swiglu_scale", gate_up.data_ptr(), gate_up.stride(0) if n > 1 else 2 * experts * ff, dense.data_ptr(),
-                      dense.stride(0) if n > 1 else dense.shape[1], n, experts, ff, out.data_ptr(), self.code, self._stream())
+                      dense.stride(0) if n > 1 else dense.shape[1], n, experts, ff, out.data_ptr(), float(limit), float(slope),
+                      self.code, self._stream())
 
     def moe_identity_add(self, y: torch.Tensor, h: torch.Tensor, dense: torch.Tensor, first: int, count: int,
                          overwrite: bool = False) -> None:
@@ -1565,11 +1698,13 @@ class Ops:
     def attention(self, q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                   block_table: torch.Tensor, page_size: int, positions: torch.Tensor, token_seq: torch.Tensor,
                   num_heads: int, num_kv_heads: int, head_dim: int, scale: float, window: Optional[int],
-                  plan: Optional["AttentionPlan"] = None) -> None:
+                  plan: Optional["AttentionPlan"] = None, keep_first: int = 0, gate: Optional[torch.Tensor] = None) -> None:
         """Causal attention of the step's queries over the paged cache.
 
         q: [n, >= H*D] rows (a view into the qkv rows), out: [n, H*D]. The query at position p
-        of sequence s sees keys max(0, p - window) .. p of s. ``plan`` carries what the faster
+        of sequence s sees keys max(0, p - window) .. p of s and, with ``keep_first``, the first
+        ``keep_first`` positions of s however far back they lie. ``gate`` [n, >= H] (a view into the
+        packed rows): head h's output is multiplied by sigmoid(gate[:, h]). ``plan`` carries what the faster
         kernels need to know about the step (see AttentionPlan); without it, or in float32, the
         general kernel runs."""
         self._act(q, "queries"); self._act(out, "attention output")
@@ -1596,16 +1731,23 @@ class Ops:
         if n == 0:
             return
         w = -1 if window is None else int(window)
+        first = 0 if window is None else max(0, int(keep_first))      # without a window every key is seen anyway
         qs = q.stride(0) if n > 1 else q.shape[1]
         os_ = out.stride(0) if n > 1 else hd
+        gs = 0
+        if gate is not None:
+            self._act(gate, "head gates")
+            if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < num_heads or gate.stride(1) != 1:
+                raise KernelLibraryError(f"attention: gates {tuple(gate.shape)} do not hold {num_heads} numbers a row")
+            gs = gate.stride(0) if n > 1 else gate.shape[1]
         if self._attention_fast(q, qs, out, os_, k_pages, v_pages, block_table, page_size, positions, token_seq,
-                                num_heads, num_kv_heads, head_dim, scale, w, plan):
+                                num_heads, num_kv_heads, head_dim, scale, w, plan, first, gate, gs):
             return
         self._note_attention("mv_attention_ref", plan, n, num_heads, num_kv_heads, head_dim, q.element_size())
         self.lib.call("mv_attention_ref", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                       positions.data_ptr(), token_seq.data_ptr(), n, num_heads, num_kv_heads, head_dim,
-                      float(scale), w, self.code, self._stream())
+                      float(scale), w, first, _ptr(gate), gs, self.code, self._stream())
 
     def _note_attention(self, entry: str, plan, n_tokens: int, H: int, Hkv: int, D: int, item: int, splits: int = 1) -> None:
         """Bytes: the keys and values of every sequence once (per key, so that the line can be priced
@@ -1765,9 +1907,11 @@ class Ops:
         return nt, kw, n_units, n_busy
 
     def _attention_fast(self, q, qs, out, os_, k_pages, v_pages, block_table, page_size, positions, token_seq,
-                        H, Hkv, D, scale, window, plan) -> bool:
+                        H, Hkv, D, scale, window, plan, first: int = 0, gate=None, gs: int = 0) -> bool:
         """The MFMA kernels, when the step and the sizes allow them."""
         if not self.use_fast_kernels or plan is None or not self.lib.has("mv_attention_decode"):
+            return False
+        if first > 0 or gate is not None:
             return False
         if D not in (64, 128) or page_size % 16 or qs % 8 or os_ % 4 or q.data_ptr() % 16 or out.data_ptr() % 8:
             return False

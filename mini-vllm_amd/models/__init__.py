@@ -3,4 +3,5 @@ from .registry import (Architecture, config_from_dict, get_architecture, load_co
 from . import qwen3  # registers "Qwen3ForCausalLM"
 from . import bolapel  # registers "Bolapel"
 from . import dutilix  # registers "Dutilix"
+from . import zedudra  # registers "Zedudra"
 from .causal_lm import CausalLM, expected_tensors

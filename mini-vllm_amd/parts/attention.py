@@ -14,7 +14,10 @@ Beyond the reference's layer the spec has, each off by default: values of anothe
 with equal ``position // chunk``, counted from the sequence's start); ``weighting = "sigmoid"``: the
 weight of a visible key is sigmoid(score * scale + score_bias[head]) and the weights are not
 normalised over the keys; ``head_gate``: head h's output is multiplied by sigmoid(W_gate x)[h], one
-number per head, read from the same packed product as q, k and v.
+number per head, read from the same packed product as q, k and v; ``keep_first`` (with a window): a
+query also sees the sequence's first ``keep_first`` positions however far back they lie, at their true
+positions; ``value_from_key``: there is no value projection, the values are the keys as projected,
+before norm and rotation. Softmax weighting with any of the last three runs ``_forward_kept``.
 """
 from __future__ import annotations
 
@@ -23,7 +26,8 @@ from typing import Dict, Optional, Tuple
 
 import torch
 
-from .base import CacheNeed, KeepAll, KeepChunks, KeepWindow, KeyValueNeed, Mixer, PartSpec, Runtime, TensorDecl, register_mixer
+from .base import (CacheNeed, KeepAll, KeepChunks, KeepWindow, KeepWindowAndFirst, KeyValueNeed, Mixer, PartSpec, Runtime,
+                   TensorDecl, register_mixer)
 
 
 @dataclass(frozen=True)
@@ -49,6 +53,8 @@ class AttentionSpec(PartSpec):
     # pages stay); empty: its own ``chunk`` alone. ``cache_keeps_all``: some reader sees all keys.
     cache_chunks: Tuple[int, ...] = ()
     cache_keeps_all: bool = False
+    keep_first: int = 0                      # with a window: the sequence's first positions stay visible
+    value_from_key: bool = False             # values = keys as projected (no value projection)
 
     @property
     def q_dim(self) -> int:
@@ -74,7 +80,13 @@ class AttentionSpec(PartSpec):
     def plain(self) -> bool:
         """The reference's layer: softmax over all keys or a window, values as large as keys."""
         return (self.weighting == "softmax" and self.chunk is None and self.value_dim in (None, self.head_dim)
-                and not self.head_gate and not self.score_bias)
+                and not self.head_gate and not self.score_bias and not self.keep_first and not self.value_from_key)
+
+    @property
+    def kept(self) -> bool:
+        """Softmax over a window (or all keys) with kept first positions, head gates or values taken from the keys."""
+        return (self.weighting == "softmax" and self.chunk is None and self.value_dim in (None, self.head_dim)
+                and not self.score_bias and not self.bias and not self.qk_norm and not self.plain)
 
 
 @register_mixer(AttentionSpec.kind)
@@ -88,7 +100,8 @@ class Attention(Mixer):
         t = {"q": TensorDecl((spec.q_dim, spec.hidden_size)), "o": TensorDecl((spec.hidden_size, spec.out_dim))}
         if not spec.shares_kv:
             t["k"] = TensorDecl((spec.kv_dim, spec.hidden_size))
-            t["v"] = TensorDecl((spec.v_dim, spec.hidden_size))
+            if not spec.value_from_key:
+                t["v"] = TensorDecl((spec.v_dim, spec.hidden_size))
         if spec.score_bias:
             t["score_bias"] = TensorDecl((spec.num_heads,), init="zeros_normal")
         if spec.head_gate:
@@ -113,7 +126,12 @@ class Attention(Mixer):
             sizes = tuple(sorted(set(spec.cache_chunks or (spec.chunk,))))
             retention = KeepAll() if spec.cache_keeps_all else KeepChunks(sizes)
         else:
-            retention = KeepAll() if (spec.window is None or spec.cache_keeps_all) else KeepWindow(spec.window)
+            if spec.window is None or spec.cache_keeps_all:
+                retention = KeepAll()
+            elif spec.keep_first > 0:
+                retention = KeepWindowAndFirst(spec.window, spec.keep_first)
+            else:
+                retention = KeepWindow(spec.window)
         return KeyValueNeed(retention=retention, num_kv_heads=spec.num_kv_heads, head_dim=spec.head_dim,
                             value_dim=spec.value_dim)
 
@@ -123,12 +141,17 @@ class Attention(Mixer):
             raise ValueError(f"{spec.num_heads} query heads are not a multiple of {spec.num_kv_heads} kv heads")
         if spec.weighting not in ("softmax", "sigmoid"):
             raise ValueError(f"attention weighting must be 'softmax' or 'sigmoid', got {spec.weighting!r}")
-        if not spec.plain and (spec.weighting != "sigmoid" or spec.bias):
-            raise NotImplementedError("chunks, a value size of its own, a score bias and head gates are built for "
-                                      "sigmoid weighting without projection biases")
+        if not spec.plain and not spec.kept and (spec.weighting != "sigmoid" or spec.bias):
+            raise NotImplementedError("chunks, a value size of its own and a score bias are built for sigmoid weighting "
+                                      "without projection biases; kept first positions, head gates and values taken from "
+                                      "the keys also for softmax weighting without biases and query/key norms")
+        if spec.keep_first < 0 or (spec.value_from_key and (spec.shares_kv or spec.v_head_dim != spec.head_dim)):
+            raise ValueError("values taken from the keys have the keys' size and a cache of their own; keep_first is >= 0")
+        if (spec.keep_first or spec.value_from_key) and not spec.kept:
+            raise NotImplementedError("kept first positions and values taken from the keys are built for softmax weighting")
         self.spec = spec
         self.rt = rt
-        parts = ["q"] if spec.shares_kv else ["q", "k", "v"]
+        parts = ["q"] if spec.shares_kv else (["q", "k"] if spec.value_from_key else ["q", "k", "v"])
         if spec.head_gate:
             parts = parts + ["head_gate"]
         dtypes = {tensors[p].dtype for p in parts}
@@ -148,7 +171,7 @@ class Attention(Mixer):
         self.rotary = position.rotary() if position is not None else None
         if position is not None and self.rotary is None and not hasattr(position, "apply"):
             raise ValueError("a position encoding must offer rotary() or apply()")
-        self.width = spec.q_dim + (0 if spec.shares_kv else spec.kv_dim + spec.v_dim)
+        self.width = spec.q_dim + (0 if spec.shares_kv else spec.kv_dim + (0 if spec.value_from_key else spec.v_dim))
         self.gate_off = self.width                        # the head gates come last in the packed rows
         if spec.head_gate:
             self.width += spec.num_heads
@@ -169,6 +192,8 @@ class Attention(Mixer):
 
     def forward(self, x: torch.Tensor, ctx, call: int, fold=None) -> torch.Tensor:
         spec, rt, ops = self.spec, self.rt, self.rt.ops
+        if spec.kept:
+            return self._forward_kept(x, ctx, call)
         if not spec.plain:
             return self._forward_sigmoid(x, ctx, call)
         n = x.shape[0]
@@ -232,3 +257,30 @@ class Attention(Mixer):
                               plan=ctx.attention_plan)
         y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
         return ops.gemm(attn, self.w_o, y, self.b_o, defer_sum=True) or y
+
+    def _forward_kept(self, x: torch.Tensor, ctx, call: int) -> torch.Tensor:
+        """Softmax weighting over a window with kept first positions, head gates, values taken from the keys."""
+        spec, rt, ops, ws = self.spec, self.rt, self.rt.ops, self.rt.workspace
+        if not isinstance(x, torch.Tensor):
+            x = x.materialize()
+        n = x.shape[0]
+        packed = ws.get("attn.qkv", (n, self.width), rt.dtype)
+        ops.gemm(x, self.w_qkv, packed)
+        kv = ctx.kv(call)
+        table, interleaved = (self.rotary if self.rotary is not None else (None, False))
+        if self.position is not None and self.rotary is None:
+            raise NotImplementedError("this attention takes its rotation from a rotary table")
+        own = not spec.shares_kv
+        held = spec.q_dim + (0 if not own else spec.kv_dim + (0 if spec.value_from_key else spec.v_dim))
+        ops.qk_norm_rope_store(
+            packed, spec.num_heads, spec.num_kv_heads, spec.head_dim, ctx.positions, ctx.token_seq,
+            None, None, spec.qk_norm_eps, table, interleaved,
+            kv.k_pages if own else None, kv.v_pages if own else None, kv.block_table if own else None, kv.page_size,
+            value_from_key=spec.value_from_key, extra_columns=self.width - held)
+        attn = ws.get("attn.out", (n, spec.out_dim), rt.dtype)
+        gate = packed[:, self.gate_off:self.gate_off + spec.num_heads] if spec.head_gate else None
+        ops.attention(packed[:, :spec.q_dim], attn, kv.k_pages, kv.v_pages, kv.block_table, kv.page_size, ctx.positions,
+                      ctx.token_seq, spec.num_heads, spec.num_kv_heads, spec.head_dim, spec.scale, spec.window,
+                      plan=ctx.attention_plan, keep_first=spec.keep_first, gate=gate)
+        y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
+        return ops.gemm(attn, self.w_o, y, defer_sum=True) or y

@@ -64,6 +64,11 @@ class Retention:
         return np.fromiter((self.first_kept_page(int(p), page_size) for p in next_positions), dtype=np.int64,
                            count=len(next_positions))
 
+    def leading_pages_kept(self, page_size: int) -> int:
+        """How many of a request's first pages stay for its whole life whatever ``first_kept_page`` says
+        (a rule whose queries also see the sequence's first positions); they are never given back."""
+        return 0
+
     def most_pages(self, length: int, page_size: int) -> Optional[int]:
         """Most pages a request of ``length`` tokens holds at one time, if the rule can tell
         (a request that needs more than its pool has is refused when it is submitted)."""
@@ -119,6 +124,32 @@ class KeepWindow(Retention):
         # while a portion runs: the window behind its first token, the portion itself, and the two
         # pages that the ends of that range may only touch
         return min(-(-length // page_size), (self.window + max(1, portion)) // page_size + 2)
+
+
+@dataclass(frozen=True)
+class KeepWindowAndFirst(Retention):
+    """The last ``window`` positions besides the query's own stay, and so do the sequence's first
+    ``first`` positions for as long as the request lives; the pages between go back to the pool."""
+    window: int = 0
+    first: int = 0
+
+    def __post_init__(self):
+        if self.window < 0 or self.first < 0:
+            raise ValueError(f"a window and the count of kept first positions must be >= 0, got {self.window}, {self.first}")
+
+    def first_kept_page(self, next_position: int, page_size: int) -> int:
+        return max(0, next_position - self.window) // page_size
+
+    def first_kept_pages(self, next_positions, page_size: int):
+        import numpy as np
+        return np.maximum(0, np.asarray(next_positions, dtype=np.int64) - self.window) // page_size
+
+    def leading_pages_kept(self, page_size: int) -> int:
+        return -(-self.first // page_size)
+
+    def most_pages_held(self, length: int, page_size: int, portion: int) -> Optional[int]:
+        return min(-(-length // page_size),
+                   (self.window + max(1, portion)) // page_size + 2 + self.leading_pages_kept(page_size))
 
 
 @dataclass(frozen=True)

@@ -76,10 +76,13 @@ class PreNormBlock(Block):
 @dataclass(frozen=True)
 class SandwichBlockSpec(PartSpec):
     """A norm in front of and behind every sublayer; ``token_shift`` mixes each row of the mixer's
-    input with the row of the token before it (``hidden_size`` is the width of those rows)."""
+    input with the row of the token before it (``hidden_size`` is the width of those rows);
+    ``input_conv_taps`` > 0 adds to each row of the mixer's input a causal convolution over time of
+    those rows, channel by channel, with that many taps."""
     kind = "sandwich"
     hidden_size: int = 0
     token_shift: bool = False
+    input_conv_taps: int = 0
 
 
 @register_block(SandwichBlockSpec.kind)
@@ -88,8 +91,10 @@ class SandwichBlock(Block):
 
     ``shift``: h[t] <- h[t] + (h[t-1] - h[t]) * mix, element by element, with the rows as the norm
     left them; the row in front of a request's first token is zero, and the last row of a step is
-    kept as the request's state (``shift.last``) for its next step. A layer without a feed-forward
-    has only the first half.
+    kept as the request's state (``shift.last``) for its next step. With an input convolution of T
+    taps instead: h[t] <- h[t] + sum_j canon[:, j] * h[t - T + 1 + j] (the last tap multiplies h[t]
+    itself), zeros in front of a request's first token; the last T - 1 rows are the request's state
+    (``conv.last``). A layer without a feed-forward has only the first half.
 
     The norm behind a sublayer, the residual add and the norm in front of the next sublayer are
     one kernel when both norms are plain scaled RMS norms (``Norm.as_scaled_rms``): the sum never
@@ -105,12 +110,19 @@ class SandwichBlock(Block):
     @classmethod
     def tensors(cls, spec: SandwichBlockSpec):
         from .base import TensorDecl
-        return {"shift": TensorDecl((spec.hidden_size,), init="zeros_normal")} if spec.token_shift else {}
+        t = {"shift": TensorDecl((spec.hidden_size,), init="zeros_normal")} if spec.token_shift else {}
+        if spec.input_conv_taps > 0:
+            t["canon"] = TensorDecl((spec.hidden_size, spec.input_conv_taps), init="zeros_normal")
+        return t
 
     @classmethod
     def state_shapes(cls, spec: SandwichBlockSpec):
         # the mixer's input row of the request's last token, in the activation type (None: the runtime's)
-        return {"shift.last": ((spec.hidden_size,), None)} if spec.token_shift else {}
+        shapes = {"shift.last": ((spec.hidden_size,), None)} if spec.token_shift else {}
+        if spec.input_conv_taps > 1:
+            # the mixer's input rows of the request's last taps - 1 tokens, as the norm left them
+            shapes["conv.last"] = ((spec.input_conv_taps - 1, spec.hidden_size), None)
+        return shapes
 
     def __init__(self, spec: SandwichBlockSpec, norms: Dict[str, Norm], mixer: Mixer, ffn: FeedForward,
                  tensors=None, rt=None):
@@ -121,6 +133,11 @@ class SandwichBlock(Block):
         self.shift = (tensors or {}).get("shift")
         if spec.token_shift and (self.shift is None or rt is None):
             raise ValueError("a block with token shift needs its 'shift' tensor and the runtime")
+        self.canon = (tensors or {}).get("canon")
+        if spec.input_conv_taps > 0 and (self.canon is None or rt is None):
+            raise ValueError("a block with an input convolution needs its 'canon' tensor and the runtime")
+        if spec.input_conv_taps > 0 and spec.token_shift:
+            raise ValueError("a block shapes its mixer's input by a token shift or by a convolution, not both")
 
     def entry_norm(self) -> Norm:
         return self.norm_in
@@ -128,15 +145,26 @@ class SandwichBlock(Block):
     def entry_part(self):
         # the rows pass through the shift first: no product takes the norm over; a block in front may
         # apply this block's shift together with its norm (``TokenShiftEntry``)
+        if self.canon is not None:
+            return InputConvEntry(self.canon)
         return TokenShiftEntry(self.shift) if self.shift is not None else None
 
+    def _conv_state(self, ctx, call: int):
+        return ctx.state(call, "conv.last") if self.spec.input_conv_taps > 1 else None
+
     def forward(self, stream: HiddenStream, ctx, call: int, next_norm: Optional[Norm] = None, next_part=None) -> None:
-        already = stream.normed is not None and len(stream.normed) > 2 and stream.normed[2] is self.shift
+        mine = self.shift if self.shift is not None else self.canon
+        already = mine is not None and stream.normed is not None and len(stream.normed) > 2 and stream.normed[2] is mine
         h = self.norm_in.forward(stream, ctx)
         if self.shift is not None and not already:
             mixed = self.rt.workspace.get("shift.out", tuple(h.shape), h.dtype)
             self.rt.ops.token_shift(h, self.shift, ctx.state(call, "shift.last"), ctx.token_seq, ctx.cu_seqlens,
                                     ctx.state_slots, mixed)
+            h = mixed
+        elif self.canon is not None and not already:
+            mixed = self.rt.workspace.get("conv.out", tuple(h.shape), h.dtype)
+            self.rt.ops.input_conv(h, self.canon, self._conv_state(ctx, call), ctx.token_seq, ctx.cu_seqlens,
+                                   ctx.state_slots, ctx.n_seqs, mixed)
             h = mixed
         y = self.mixer.forward(h, ctx, call)
         last = self.ffn is None
@@ -154,6 +182,8 @@ class SandwichBlock(Block):
             y = y.materialize()
         out_form = norm_out.as_scaled_rms()
         next_form = norm_next.as_scaled_rms() if norm_next is not None else None
+        if out_form is None and self._close_grouped(stream, ctx, y, norm_out, norm_next, call, next_part):
+            return
         if out_form is None:
             tmp = self.rt.workspace.get("sandwich.delta", tuple(y.shape), y.dtype)
             norm_out.apply(y, tmp)
@@ -173,6 +203,42 @@ class SandwichBlock(Block):
             stream.normed = None
         else:
             stream.normed = (norm_next, rows, next_part.mix) if shift is not None else (norm_next, rows)
+
+
+    def _close_grouped(self, stream: HiddenStream, ctx, y, norm_out: Norm, norm_next: Optional[Norm], call: int,
+                       next_part) -> bool:
+        """The same in one kernel for norms in groups (``as_grouped_rms``); in a step of single tokens the next
+        block's input convolution rides along. False, having done nothing, when the norms are of another form."""
+        form = getattr(norm_out, "as_grouped_rms", None)
+        if form is None:
+            return False
+        wa, eps_a, groups = form()
+        nxt = getattr(norm_next, "as_grouped_rms", None) if norm_next is not None else None
+        rows = second = conv = None
+        if nxt is not None and nxt()[2] == groups:
+            wb, eps_b, _ = nxt()
+            second = (wb, eps_b)
+            rows = self.rt.workspace.get("normed", tuple(y.shape), y.dtype)
+        plan = getattr(ctx, "attention_plan", None)
+        if rows is not None and isinstance(next_part, InputConvEntry) and plan is not None and plan.decode_only:
+            taps = next_part.taps
+            state = ctx.state(call + 1, "conv.last") if taps.shape[1] > 1 else None    # the block that runs next is call + 1
+            conv = (taps, state, ctx.token_seq, ctx.state_slots)
+        self.rt.ops.group_norm_add_norm(y, (wa, eps_a), stream.resid, second, rows, groups, conv=conv)
+        stream.delta = None
+        if rows is None:
+            stream.normed = None
+        else:
+            stream.normed = (norm_next, rows, next_part.taps) if conv is not None else (norm_next, rows)
+        return True
+
+
+class InputConvEntry:
+    """What a sandwich block with an input convolution offers the block in front of it: the taps, so that
+    its rows can leave that block's last kernel with the convolution applied."""
+
+    def __init__(self, taps: torch.Tensor):
+        self.taps = taps
 
 
 class TokenShiftEntry:

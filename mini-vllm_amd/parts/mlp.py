@@ -58,3 +58,42 @@ class SwiGLU(FeedForward):
         # (the sums of a product whose K was split may be left to the next norm, or the residual add and
         # that norm folded into the product)
         return ops.gemm(act, self.w_down, y, defer_sum=True, fold=fold) or y
+
+
+@dataclass(frozen=True)
+class XIELUSpec(PartSpec):
+    """Two projections with the xIELU activation between them: y = Wd act(Wu x), where
+    act(z) = a_pos z^2 + z / 2 for z > 0 and a_neg (exp(z) - 1 - z) + z / 2 for z <= 0, with
+    a_pos = softplus(p) and a_neg = 1/2 + softplus(q) from the layer's two stored numbers (p, q)."""
+    kind = "xielu_mlp"
+    hidden_size: int = 0
+    intermediate_size: int = 0
+
+
+@register_feed_forward(XIELUSpec.kind)
+class XIELUFeedForward(FeedForward):
+    spec_class = XIELUSpec
+
+    @classmethod
+    def tensors(cls, spec: XIELUSpec) -> Dict[str, TensorDecl]:
+        return {"up": TensorDecl((spec.intermediate_size, spec.hidden_size)),
+                "down": TensorDecl((spec.hidden_size, spec.intermediate_size)),
+                "act": TensorDecl((2,), init="zeros_normal")}
+
+    def __init__(self, spec: XIELUSpec, tensors: Dict[str, torch.Tensor], rt: Runtime):
+        self.spec, self.rt = spec, rt
+        self.w_up, self.w_down = tensors["up"], tensors["down"]
+        # the two constants of the activation, once, in float32 (they belong to the weights, not to a step)
+        pq = torch.nn.functional.softplus(tensors["act"].to(torch.float32)).tolist()
+        self.a_pos, self.a_neg = float(pq[0]), 0.5 + float(pq[1])
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        spec, rt, ops = self.spec, self.rt, self.rt.ops
+        if not isinstance(x, torch.Tensor):
+            x = x.materialize()
+        n = x.shape[0]
+        act = rt.workspace.get("ffn.act", (n, spec.intermediate_size), rt.dtype)
+        ops.gemm(x, self.w_up, act)
+        ops.xielu(act, self.a_pos, self.a_neg, act)
+        y = rt.workspace.get("ffn.out", (n, spec.hidden_size), rt.dtype)
+        return ops.gemm(act, self.w_down, y, defer_sum=True) or y

@@ -24,6 +24,12 @@ of eight 12.2 against 13.4), and lose or draw elsewhere (0.6B-sized layers at ei
 2.4 ms; a prompt of 2,048 tokens 440 against 465 us a layer at 0.6B sizes, but 186 against 151 ms for the
 whole prompt at 8B sizes), so the spec's thresholds send only the former there. Either way everything is decided on the device;
 nothing about a step's routing reaches the host, so steps replay from graphs.
+
+Options of the spec, each with the default that gives the above: ``scoring`` "sigmoid" scores every router
+output by sigmoid(z) on its own; ``group_worth`` "top2" ranks a group by the sum of its two largest choices
+instead of its largest; ``normalize`` False uses the chosen scores themselves as weights; ``activation``
+"clamped" replaces the gated SiLU pair by g = min(gate, limit), u = clamp(up, -limit, limit),
+g * sigmoid(gate_slope * g) * (u + 1).
 """
 from __future__ import annotations
 
@@ -53,6 +59,12 @@ class RoutedExpertsSpec(PartSpec):
     grouped: bool = True
     grouped_max_rows: float = 2.0
     grouped_min_weight: int = 4 * 1024 * 1024
+    scoring: str = "softmax"             # or "sigmoid"
+    group_worth: str = "max"             # or "top2": the sum of a group's two largest choices
+    normalize: bool = True               # False: the weights are the chosen scores as they are
+    activation: str = "swiglu"           # or "clamped" (with ``limit`` and ``gate_slope``)
+    limit: float = 0.0
+    gate_slope: float = 1.702
 
     @property
     def router_outputs(self) -> int:
@@ -79,6 +91,10 @@ class RoutedExperts(FeedForward):
         if spec.num_experts < 0 or spec.identity_experts < 0 or E < 1 or spec.groups < 1 or E % spec.groups \
                 or not (1 <= spec.keep_groups <= spec.groups) or not (1 <= spec.top <= E // spec.groups * spec.keep_groups):
             raise ValueError(f"routed experts: bad sizes {spec}")
+        if spec.scoring not in ("softmax", "sigmoid") or spec.group_worth not in ("max", "top2") \
+                or spec.activation not in ("swiglu", "clamped") or (spec.activation == "clamped" and not spec.limit > 0):
+            raise ValueError(f"routed experts: unknown scoring, group worth or activation, or a clamped pair without a "
+                             f"positive limit: {spec}")
         self.spec, self.rt = spec, rt
         self.w_router = tensors["router"]
         self.correction = tensors.get("correction")
@@ -95,7 +111,7 @@ class RoutedExperts(FeedForward):
     def wants_grouped(self, n: int) -> bool:
         """Whether a step of n rows computes the chosen pairs only (where the kernels take the sizes)."""
         spec = self.spec
-        return (spec.grouped and n * spec.top < spec.grouped_max_rows * spec.num_experts
+        return (spec.grouped and spec.activation == "swiglu" and n * spec.top < spec.grouped_max_rows * spec.num_experts
                 and spec.expert_size * spec.hidden_size >= spec.grouped_min_weight)
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
@@ -108,7 +124,8 @@ class RoutedExperts(FeedForward):
         dense = ws.get("moe.dense", (n, E), torch.float32)
         ids = ws.get("moe.ids", (n, spec.top), torch.int32)
         weights = ws.get("moe.weights", (n, spec.top), torch.float32)
-        ops.moe_route(logits, self.correction, spec.groups, spec.keep_groups, spec.top, spec.weight_sum_eps, dense, ids, weights)
+        ops.moe_route(logits, self.correction, spec.groups, spec.keep_groups, spec.top, spec.weight_sum_eps, dense, ids, weights,
+                      scoring=spec.scoring, group_worth=spec.group_worth, normalize=spec.normalize)
         y = ws.get("ffn.out", (n, spec.hidden_size), rt.dtype)
         if n_e and ops.use_fast_kernels and self.wants_grouped(n):
             # the chosen (token, expert) pairs only: sorted by expert on the device, tiles of 64 rows through MFMA
@@ -121,7 +138,10 @@ class RoutedExperts(FeedForward):
             gu = ws.get("moe.gate_up", (n, 2 * n_e * F), rt.dtype)
             ops.gemm(x, self.w_gate_up, gu)
             act = ws.get("moe.act", (n, n_e * F), rt.dtype)
-            ops.moe_swiglu_scale(gu, dense, n_e, F, act)
+            if spec.activation == "clamped":
+                ops.moe_swiglu_scale(gu, dense, n_e, F, act, limit=spec.limit, slope=spec.gate_slope)
+            else:
+                ops.moe_swiglu_scale(gu, dense, n_e, F, act)
             ops.gemm(act, self.w_down, y)
         if spec.identity_experts or not n_e:
             ops.moe_identity_add(y, x, dense, n_e, spec.identity_experts, overwrite=not n_e)

@@ -96,3 +96,53 @@ class RMSNorm(Norm):
 
     def apply(self, x: torch.Tensor, out: torch.Tensor) -> None:
         self.rt.ops.rmsnorm(x, self.weight, self.spec.eps, out, unit_offset=self.spec.unit_offset)
+
+
+@dataclass(frozen=True)
+class GroupRMSNormSpec(PartSpec):
+    """RMS norm in groups: a row is cut into ``groups`` equal runs of neighbouring columns, each run is
+    divided by sqrt(mean of its squares + eps), and the whole row is multiplied by the weight."""
+    kind = "group_rmsnorm"
+    size: int = 0
+    eps: float = 1e-6
+    groups: int = 1
+
+
+@register_norm(GroupRMSNormSpec.kind)
+class GroupRMSNorm(Norm):
+    spec_class = GroupRMSNormSpec
+
+    @classmethod
+    def tensors(cls, spec: GroupRMSNormSpec) -> Dict[str, TensorDecl]:
+        return {"weight": TensorDecl((spec.size,), init="ones_normal")}
+
+    def __init__(self, spec: GroupRMSNormSpec, tensors: Dict[str, torch.Tensor], rt: Runtime):
+        if spec.groups < 1 or spec.size % spec.groups:
+            raise ValueError(f"rows of {spec.size} columns do not form {spec.groups} equal groups")
+        self.spec = spec
+        self.rt = rt
+        self.weight = tensors["weight"]
+
+    def forward(self, stream: HiddenStream, ctx, rows: Optional[torch.Tensor] = None,
+                tag: str = "normed") -> torch.Tensor:
+        ready, stream.normed = stream.normed, None
+        if ready is not None and ready[0] is self and rows is None and stream.delta is None:
+            return ready[1]                # the kernel that made the residual has run this norm already
+        if stream.weighted is not None:
+            raise RuntimeError("the stream holds rows that were prepared for another norm")
+        delta = stream.delta
+        if delta is not None and not isinstance(delta, torch.Tensor):
+            delta = delta.materialize()
+        n = stream.resid.shape[0] if rows is None else rows.numel()
+        out = self.rt.workspace.get(tag, (n, self.spec.size), self.rt.dtype)
+        self.rt.ops.group_norm(self.weight, self.spec.eps, self.spec.groups, out, resid=stream.resid, delta=delta, rows=rows)
+        if rows is None:
+            stream.delta = None
+        return out
+
+    def as_grouped_rms(self):
+        """(weight, eps, groups): the form the fused norm + add + norm kernel computes itself."""
+        return self.weight, self.spec.eps, self.spec.groups
+
+    def apply(self, x: torch.Tensor, out: torch.Tensor) -> None:
+        self.rt.ops.group_norm(self.weight, self.spec.eps, self.spec.groups, out, x=x)
