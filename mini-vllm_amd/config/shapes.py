@@ -28,10 +28,12 @@ def named_shapes() -> Dict[str, Dict[str, Any]]:
     shapes = {name: qwen3_shape(name) for name in QWEN3_SHAPES}
     shapes["bolapel-tiny"] = bolapel_tiny_shape()
     shapes["dutilix-tiny"] = dutilix_tiny_shape()
+    shapes["zedudra-tiny"] = zedudra_tiny_shape()
     for name in QWEN3_SHAPES:
         if name != "tiny":
             shapes[f"bolapel-{name}"] = bolapel_shape(name)
             shapes[f"dutilix-{name}"] = dutilix_shape(name)
+            shapes[f"zedudra-{name}"] = zedudra_shape(name)
     return shapes
 
 
@@ -135,3 +137,40 @@ def dutilix_tiny_shape() -> Dict[str, Any]:
                         "mixer": {"heads": 4, "dim": 12, "rot_dim": 4, "vdim": 8, "q_rank": 24, "kv_rank": 16, "scale": 0.25,
                                   "rot": {"dims": 4, "base": 10000.0}}},
                        {"type": "mlstm", "mixer": {"heads": 2, "dim": 16, "vdim": 24, "gate_cap": 12.0}, "mlp": None}]}
+
+
+def zedudra_shape(name: str, layers: int = None, window: int = 1024, keep_first: int = 64, experts: int = 32, top: int = 4,
+                  groups: int = 4, keep: int = 2, taps: int = 4, norm_groups: int = 4, limit: float = 7.0,
+                  dense_every: int = 2) -> Dict[str, Any]:
+    """A Zedudra configuration with the width, vocabulary, head counts, head size and number of layers of the named
+    Qwen3 shape: every layer is attention over a window of ``window`` positions beside the first ``keep_first``, with a
+    rotation over half of each head; every ``dense_every``-th feed-forward (from the first) is dense at the shape's
+    width, the others are mixtures of ``experts`` experts of which ``top`` are used, each 1/top of the dense width.
+    For random-weights models at sizes that resemble a real model's layers."""
+    q = QWEN3_SHAPES[name]
+    n = layers or q["num_hidden_layers"]
+    hid, hd = q["hidden_size"], q["head_dim"]
+    dense = {"kind": "dense", "ff": q["intermediate_size"]}
+    sparse = {"kind": "moe", "expert": {"ff": q["intermediate_size"] // top, "limit": limit},
+              "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}}}
+    mixer = {"heads": q["num_attention_heads"], "kv_heads": q["num_key_value_heads"], "dim": hd, "vdim": hd,
+             "scale": hd ** -0.5, "mask": {"size": window, "keep_first": keep_first},
+             "rot": {"dims": hd // 2, "base": q["rope_theta"]}}
+    out = [{"type": "attention", "mixer": dict(mixer), "mlp": dense if i % dense_every == 0 else sparse} for i in range(n)]
+    return {"architecture": "Zedudra", "vocab": q["vocab_size"], "width": hid, "layers": out,
+            "norm": {"eps": q["rms_norm_eps"], "groups": norm_groups}, "canon": {"taps": taps},
+            "embedding": {"scale": float(hid) ** 0.5}}
+
+
+def zedudra_tiny_shape() -> Dict[str, Any]:
+    """A Zedudra model of a few thousand weights: a dense layer, a routed layer that runs twice, a layer without
+    feed-forward."""
+    mixer = {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 16, "scale": 0.25, "mask": {"size": 24, "keep_first": 4},
+             "rot": {"dims": 8, "base": 10000.0}}
+    moe = {"kind": "moe", "expert": {"ff": 32, "limit": 2.0}, "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}
+    return {"architecture": "Zedudra", "vocab": 256, "width": 64, "norm": {"eps": 1e-5, "groups": 2}, "canon": {"taps": 3},
+            "embedding": {"scale": 8.0},
+            "layers": [{"type": "attention", "mixer": dict(mixer), "mlp": {"kind": "dense", "ff": 96}},
+                       {"type": "attention", "mixer": dict(mixer), "mlp": moe},
+                       {"type": "attention", "mixer": dict(mixer), "mlp": moe, "weights_of": 1},
+                       {"type": "attention", "mixer": dict(mixer, kv_heads=4), "mlp": None}]}

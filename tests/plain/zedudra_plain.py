@@ -62,6 +62,13 @@ def visible(i: int, j: int, window: int, keep_first: int) -> bool:
     return j <= i and (i - j < window or j < keep_first)
 
 
+def visibility(start: int, n: int, window: int, keep_first: int) -> torch.Tensor:
+    """bool [n, start + n]: row t is the query at position start + t, column j the key at position j."""
+    i = torch.arange(start, start + n)[:, None]
+    j = torch.arange(start + n)[None, :]
+    return (j <= i) & ((i - j < window) | (j < keep_first))
+
+
 def attention_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, m: dict, start: int = 0,
                     past: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, rnd=None):
     """h [n, width]: rows at positions start .. start + n - 1. ``past`` = (rotated keys, values) of the positions
@@ -83,15 +90,13 @@ def attention_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, m:
         k = torch.cat([past[0], k], dim=0)
         v = torch.cat([past[1], v], dim=0)
     size, first = m["mask"]["size"], m["mask"].get("keep_first", 0)
+    allowed = visibility(start, n, size, first)                      # [n, start + n]
     out = torch.zeros(n, H, Dv, dtype=h.dtype)
-    for t in range(n):
-        i = start + t
-        keys = [j for j in range(i + 1) if visible(i, j, size, first)]
-        for hd in range(H):
-            g = hd // (H // G)
-            s = (k[keys, g] @ q[t, hd]) * m["scale"]
-            p = torch.softmax(s, dim=0)
-            out[t, hd] = p @ v[keys, g]
+    for hd in range(H):
+        g = hd // (H // G)
+        s = (q[:, hd] @ k[:, g].T) * m["scale"]                      # [n, start + n]
+        s = torch.where(allowed, s, torch.full_like(s, float("-inf")))
+        out[:, hd] = torch.softmax(s, dim=-1) @ v[:, g]
     out = rnd(out * gate[:, :, None]).reshape(n, H * Dv)
     return out @ w[prefix + "o"].T, (k, v)
 
@@ -155,6 +160,10 @@ def moe_ff(h: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, f: dict, rn
     return out
 
 
+def round_to_bfloat16(t: torch.Tensor) -> torch.Tensor:
+    return t.to(torch.bfloat16).to(t.dtype)
+
+
 def weight_layer(cfg: dict, i: int) -> int:
     """The layer whose tensors layer i uses."""
     j = cfg["layers"][i].get("weights_of")
@@ -176,8 +185,10 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int], start: int
         p = f"l{weight_layer(cfg, i)}."
         st = state[i] or {}
         h = rnd(grouped_rms_norm(x, w[p + "norm1"], groups, eps))
-        h, conv = input_conv(h, w[p + "canon1"], st.get("conv"))
-        h = rnd(h)
+        conv = None
+        if p + "canon1" in w:                        # (a model without the convolution stores no taps)
+            h, conv = input_conv(h, w[p + "canon1"], st.get("conv"))
+            h = rnd(h)
         y, kv = attention_mixer(h, w, p + "mix.", layer["mixer"], start, st.get("kv"), rnd)
         x = x + grouped_rms_norm(rnd(y), w[p + "norm1b"], groups, eps)
         f = layer.get("mlp")
