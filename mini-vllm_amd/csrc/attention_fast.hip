@@ -22,7 +22,10 @@
 //
 // Layouts: K[page][kv_head][slot][d], V[page][kv_head][d][slot]; the page size is a multiple of
 // 16. Keys outside the range (above the query's position, or more than `window` below it) get
-// probability zero; value slots that were never written are read as zero.
+// probability zero; value slots that were never written are read as zero. With `kept.first` > 0
+// (a window, finished queries) the sequence's first positions stay visible however far back they lie:
+// the blocks that hold them are dealt out in front of the window's blocks, the blocks between are
+// never touched. With `kept.gate`, head h's output is multiplied by sigmoid(gate[token][h]).
 #include "dispatch.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -111,6 +114,12 @@ __device__ __forceinline__ void prepare_head_spread(const uint16_t* raw, int j, 
 
 #define AF_MAX_SPLITS 64
 
+struct KeptArgs {
+    int first;              // kept first positions (0: none)
+    const bf16* gate;       // rows of at least H values, or null
+    long gate_stride;
+};
+
 // OCC workgroups are to share a compute unit (W / 4 waves of each on every SIMD): the register budget.
 // OCC 2 is for grids larger than the chip, which do not split the keys (nsplit 1): that variant
 // leaves the code of the splits out and keeps its registers for the stream of keys.
@@ -127,7 +136,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
                       const int* __restrict__ block_table, int bt_width, int page_size,
                       const int* __restrict__ positions, const int* __restrict__ cu_seqlens, int n_seqs,
                       int H, int Hkv, float scale, int window, float* __restrict__ partials,
-                      int* __restrict__ counters, int nsplit, int max_pages, FusedInput fz) {
+                      int* __restrict__ counters, int nsplit, int max_pages, FusedInput fz, KeptArgs kept) {
     constexpr int DS = D / 32;
     constexpr int DT = D / 16;
     constexpr int NT = 1;      // column tiles of a wave (the group's heads fit one tile)
@@ -244,6 +253,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         col_head[ct] = kvh * G + (col_ok[ct] ? col % G : 0);
         col_pos[ct] = col_ok[ct] ? (FUSED ? pos0 : positions[col_tok[ct]]) : -1;   // FUSED: one token, one position
         col_lo[ct] = (window >= 0 && col_pos[ct] - window > 0) ? col_pos[ct] - window : 0;
+        if (!FUSED && kept.first >= col_lo[ct]) col_lo[ct] = 0;   // the kept positions reach the window: every key from 0 on
         if (col_ok[ct]) {
             hi_w = col_pos[ct] > hi_w ? col_pos[ct] : hi_w;
             lo_w = col_lo[ct] < lo_w ? col_lo[ct] : lo_w;
@@ -282,7 +292,15 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
     }
 
     // ---- the 32-key blocks of this wave: b_begin, b_begin + b_step, ... below b_end
-    const int b0 = hi_w >= 0 ? lo_w / 32 : 0, b1 = hi_w >= 0 ? hi_w / 32 : -1;
+    // With kept first positions in front of the window (nf blocks of them) the blocks are counted as if the
+    // window's first block followed the last kept one: block number v of the walk is block v of the cache
+    // below nf and block v + shift from there on.
+    const int kept_first = FUSED ? 0 : kept.first;
+    const int rb0 = hi_w >= 0 ? lo_w / 32 : 0;
+    const int nf = (kept_first > 0 && rb0 > 0) ? ((kept_first + 31) / 32 < rb0 ? (kept_first + 31) / 32 : rb0) : 0;
+    const int shift = nf > 0 ? rb0 - nf : 0;
+    auto cache_block = [&](int v) { return v < nf ? v : v + shift; };
+    const int b0 = nf > 0 ? 0 : rb0, b1 = hi_w >= 0 ? hi_w / 32 - shift : -1;
     const int b_step = nsplit * W;
     const int b_end = b1 + 1;
     int b_begin = split * W + wave;
@@ -322,7 +340,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         n_cached = bt_width < max_pages ? bt_width : max_pages;
         if (n_cached > AF_MAX_CACHED_PAGES) n_cached = AF_MAX_CACHED_PAGES;
     } else {
-        p_first = (32 * b0) / page_size;
+        p_first = (32 * rb0) / page_size;          // (pages of kept first positions in front of it are looked up in place)
         const int p_last = hi_w >= 0 ? hi_w / page_size : -1;
         n_cached = p_last - p_first + 1;
         if (n_cached > AF_MAX_CACHED_PAGES) n_cached = AF_MAX_CACHED_PAGES;
@@ -334,7 +352,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
     auto page_of = [&](int pidx) -> int {
         if (pidx >= bt_width) return -1;
         const int rel = pidx - p_first;
-        return rel < n_cached ? sh_pages[rel] : bt[pidx];
+        return (rel >= 0 && rel < n_cached) ? sh_pages[rel] : bt[pidx];
     };
     // Which keys a lane's operand slots hold: row rho of score tile t is key 8 (rho / 4) + 4 t + rho % 4 of
     // the block, so that after the first product lane group g holds the probabilities of keys 8 g ..
@@ -353,7 +371,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         int slot0[2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const int key0 = 32 * b + 16 * h;
+            const int key0 = 32 * cache_block(b) + 16 * h;
             const int pidx = key0 / page_size;
             op.page[h] = (b < b_end && key0 <= hi_w) ? (given ? (h ? pg1 : pg0) : page_of(pidx)) : -1;
             slot0[h] = key0 - pidx * page_size;
@@ -386,7 +404,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
         }
     };
     auto compute = [&](int b, Operands& op) {
-        const int base = 32 * b;
+        const int base = 32 * cache_block(b);
         if (FUSED && owns_new && b == b_new) {   // the newest key and value come from the registers
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
@@ -416,7 +434,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int key = base + 8 * g + 4 * t + r;
-                const bool ok = v_live && col_ok[0] && key <= col_pos[0] && key >= col_lo[0];
+                const bool ok = v_live && col_ok[0] && key <= col_pos[0] && (key >= col_lo[0] || key < kept_first);
                 p[t][r] = ok ? sacc[r] * sc_mul : -INFINITY;
             }
         }
@@ -539,6 +557,9 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
     }
     float* prow = nullptr;
     bf16* orow = nullptr;
+    float gate_mul = 1.f;
+    if (col_ok[0] && kept.gate != nullptr)
+        gate_mul = 1.f / (1.f + __expf(-to_f(kept.gate[(size_t)col_tok[0] * kept.gate_stride + col_head[0]])));
     if (col_ok[0]) {
         prow = partials ? partials + (((size_t)col_tok[0] * H + col_head[0]) * nsplit + split) * (D + 2) : nullptr;
         orow = out + (size_t)col_tok[0] * out_stride + (size_t)col_head[0] * D;
@@ -564,7 +585,7 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
                 }
                 const int d0 = 16 * (half * HALF + dt) + 4 * g;
                 if (OCC != 1 || nsplit == 1) {
-                    const float inv = 1.f / l_fin;
+                    const float inv = gate_mul / l_fin;
                     uint2 packed;
                     packed.x = f32x2_to_bf16x2_bits(o[0] * inv, o[1] * inv);
                     packed.y = f32x2_to_bf16x2_bits(o[2] * inv, o[3] * inv);
@@ -637,7 +658,8 @@ attention_decode_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restr
                 a += w * v[u];
             }
         }
-        out[(size_t)tok * out_stride + (size_t)head * D + d] = from_f<bf16>(l > 0.f ? a / l : 0.f);
+        const float gm = kept.gate != nullptr ? 1.f / (1.f + __expf(-to_f(kept.gate[(size_t)tok * kept.gate_stride + head]))) : 1.f;
+        out[(size_t)tok * out_stride + (size_t)head * D + d] = from_f<bf16>(l > 0.f ? gm * a / l : 0.f);
     }
 #undef AF_PEEK
 }
@@ -647,11 +669,11 @@ static void launch_decode(dim3 grid, hipStream_t stream, const void* q, long q_s
                           const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
                           int page_size, const int* positions, const int* cu_seqlens, int n_seqs, int H, int Hkv,
                           float scale, int window, float* partials, int* counters, int nsplit, int max_pages,
-                          const FusedInput& fz) {
+                          const FusedInput& fz, const KeptArgs& kept) {
     hipLaunchKernelGGL((attention_decode_kernel<D, W, FUSED, OCC>), grid, dim3(64 * W), 0, stream, (const bf16*)q, q_stride,
                        (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table, bt_width,
                        page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window, partials, counters, nsplit, max_pages,
-                       fz);
+                       fz, kept);
 }
 
 static int check_common(const char* what, long q_stride, long out_stride, int page_size, int bt_width, int H, int Hkv,
@@ -670,7 +692,10 @@ static int decode_common(bool fused, const FusedInput& fz, const void* q, long q
                          const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
                          int page_size, const int* positions, const int* cu_seqlens, int n_seqs, int H, int Hkv, int D,
                          float scale, int window, float* partials, int* counters, int nsplit, int max_pages, int waves,
-                         const int* token_seq, hipStream_t stream) {
+                         const int* token_seq, hipStream_t stream, KeptArgs kept = KeptArgs{0, nullptr, 0}) {
+    MV_REQUIRE(kept.first >= 0 && (kept.gate == nullptr || kept.gate_stride >= H) && (!fused || kept.first == 0),
+               "attention_decode: bad count of kept first positions (none with raw rows) or gate rows too short");
+    if (window < 0) kept.first = 0;          // without a window every key is seen anyway
     MV_REQUIRE(H / Hkv <= 16, "attention_decode: %d query heads per kv head exceed 16", H / Hkv);
     MV_REQUIRE(nsplit >= 1 && nsplit <= AF_MAX_SPLITS && (nsplit == 1 || (partials != nullptr && counters != nullptr)),
                "attention_decode: bad split count %d or missing work area or counters", nsplit);
@@ -690,13 +715,13 @@ static int decode_common(bool fused, const FusedInput& fz, const void* q, long q
             if (occ == 2) {                                                                                       \
                 launch_decode<DD, WW, FF, 2>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages,        \
                                              block_table, bt_width, page_size, positions, cu_seqlens, n_seqs, H,  \
-                                             Hkv, scale, window, part, counters, nsplit, max_pages, fz);          \
+                                             Hkv, scale, window, part, counters, nsplit, max_pages, fz, kept);    \
                 break;                                                                                            \
             }                                                                                                     \
         }                                                                                                         \
         launch_decode<DD, WW, FF, 1>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table,   \
                                      bt_width, page_size, positions, cu_seqlens, n_seqs, H, Hkv, scale, window,   \
-                                     part, counters, nsplit, max_pages, fz);                                      \
+                                     part, counters, nsplit, max_pages, fz, kept);                                \
     } while (0)
     if (fused) {
         MV_REQUIRE(waves == 4, "attention_decode_fused: %d waves per workgroup (4 only)", waves);
@@ -723,11 +748,12 @@ extern "C" int mv_attention_decode(const void* q, long q_stride, void* out, long
                                    const void* v_pages, const int* block_table, int bt_width, int page_size,
                                    const int* positions, const int* cu_seqlens, int n_seqs, int H, int Hkv, int D,
                                    float scale, int window, float* partials, int* counters, int nsplit,
-                                   int max_pages, int waves, const int* token_seq, hipStream_t stream) {
+                                   int max_pages, int waves, const int* token_seq, int first, const void* gate,
+                                   long gate_stride, hipStream_t stream) {
     if (int rc = check_common("attention_decode", q_stride, out_stride, page_size, bt_width, H, Hkv, D)) return rc;
     return decode_common(false, FusedInput{}, q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width,
                          page_size, positions, cu_seqlens, n_seqs, H, Hkv, D, scale, window, partials, counters, nsplit,
-                         max_pages, waves, token_seq, stream);
+                         max_pages, waves, token_seq, stream, KeptArgs{first, (const bf16*)gate, gate_stride});
 }
 
 // The same for a decode step whose queries, keys and values are still the raw rows of the

@@ -65,11 +65,17 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // max(start of its chunk, position - window, 0), chunks being runs of `chunk` positions counted from
 // the sequence's start (chunk <= 0: none). At the end head h's row is multiplied by
 // sigmoid(gate[token][h]) when gates are given.
+//
+// Softmax weights take two of these too: the gates (head h's row times sigmoid(gate[token][h])), and
+// `first`: beside its window a column sees the sequence's first `first` positions however far back they
+// lie. The blocks that hold them are walked in front of the window's blocks (block_of), and the blocks
+// between, whose pages may have gone back to the pool, are never touched.
 struct SigmoidArgs {
     int chunk;
     const float* bias;         // [H] or null
     const bf16* gate;          // rows of at least H values, or null
     long gate_stride;
+    int first;                 // kept first positions (softmax weights with a window; 0: none)
 };
 
 template <int D, int NT, int KW, bool SIG = false>
@@ -162,6 +168,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         col_head[ct] = kvh * G + (col_ok[ct] ? col % G : 0);
         col_pos[ct] = col_ok[ct] ? positions[col_tok[ct]] : -1;
         col_lo[ct] = (window >= 0 && col_pos[ct] - window > 0) ? col_pos[ct] - window : 0;
+        if (!SIG && sig.first >= col_lo[ct]) col_lo[ct] = 0;      // the kept positions reach the window: every key from 0 on
         col_bias[ct] = 0.f;
         if constexpr (SIG) {
             if (sig.chunk > 0 && col_pos[ct] >= 0) {
@@ -202,6 +209,9 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
     lo_g = __builtin_amdgcn_readfirstlane(lo_g);
     if (hi_g < 0) return;
     const int b0 = lo_g / 32, b1 = hi_g / 32;
+    // blocks of kept first positions that lie in front of every column's window (none with SIG or without kept positions)
+    const int kept_first = SIG ? 0 : sig.first;
+    const int nf = (kept_first > 0 && b0 > 0) ? ((kept_first + 31) / 32 < b0 ? (kept_first + 31) / 32 : b0) : 0;
 
     float m_run[NT], l_run[NT];
     floatx4_t acc_o[NT][DT];
@@ -264,8 +274,12 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
         k_lane = k_head + (size_t)hk * D * sizeof(bf16) + k_off[0];
         v_lane = v_head + (size_t)hv * sizeof(bf16) + v_off[0];
     }
-    // round j of the walk: key group kg has block b0 + j * KW + kg
-    auto block_of = [&](int j) { return b0 + j * KW + kg; };
+    // round j of the walk: key group kg has the (j * KW + kg)-th block of the walk, the nf blocks of kept
+    // first positions, then b0, b0 + 1, ...
+    auto block_of = [&](int j) {
+        const int idx = j * KW + kg;
+        return idx < nf ? idx : b0 + idx - nf;
+    };
     auto page_ids = [&](int j) {
         int b = block_of(j);
         b = b < b1 ? b : b1;    // past the unit's range: some valid entry (the block is not fetched)
@@ -348,9 +362,12 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
 
     // the blocks the wave has anything to do with, and those of them that need no mask
     const int bw_hi = (hi_w >> 5) < b1 ? (hi_w >> 5) : b1, bw_lo = lo_w >> 5;
+    // (kept first positions lie in blocks below kept_blocks, whether the unit walks them in front of its
+    // range, nf > 0, or they belong to the range because some other wave's window still reaches them)
+    const int kept_blocks = (kept_first + 31) >> 5;
     auto wanted = [&](int j) {
         const int b = block_of(j);
-        return b <= bw_hi && b >= bw_lo;
+        return b <= bw_hi && (b >= bw_lo || b < kept_blocks);
     };
     const int bm_hi = (wave_full && full_hi >= 31) ? (full_hi - 31) >> 5 : -1, bm_lo = (full_lo + 31) >> 5;
     // The operands of a block come from LDS in two parts (keys, values). The walk of four waves asks
@@ -408,7 +425,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int key = base + 8 * g + 4 * t + r;
-                        const bool ok = col_ok[ct] && key <= col_pos[ct] && key >= col_lo[ct];
+                        const bool ok = col_ok[ct] && key <= col_pos[ct] && (key >= col_lo[ct] || key < kept_first);
                         p[ct][t][r] = ok ? p[ct][t][r] : -INFINITY;
                     }
         }
@@ -471,7 +488,7 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
                 acc_o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vo.vop[dt].v, pop[ct].v, acc_o[ct][dt], 0, 0, 0);
     };
 
-    const int rounds = (b1 - b0 + KW) / KW;    // the same for every wave: they meet at the barriers
+    const int rounds = (nf + b1 - b0 + KW) / KW;    // the same for every wave: they meet at the barriers
     PageIds ids_a, ids_b;
     KOps k_even, k_odd;
     VOps vals;
@@ -652,6 +669,10 @@ attention_prefill_kernel(const bf16* __restrict__ q, long q_stride, bf16* __rest
             }
         } else {
             inv = 1.f / l_run[ct];
+            if (sig.gate != nullptr) {
+                const float z = to_f(sig.gate[(size_t)col_tok[ct] * sig.gate_stride + col_head[ct]]);
+                inv *= 1.f / (1.f + __expf(-z));
+            }
         }
         bf16* orow = out + (size_t)col_tok[ct] * out_stride + (size_t)col_head[ct] * D;
 #pragma unroll
@@ -674,7 +695,7 @@ template <int D, int NT, int KW, bool SIG = false>
 static int launch_prefill(dim3 grid, hipStream_t stream, const void* q, long q_stride, void* out, long out_stride,
                           const void* k_pages, const void* v_pages, const int* block_table, int bt_width,
                           int page_size, int page_shift, const int* positions, const int* cu_seqlens, int n_seqs,
-                          int H, int Hkv, float scale, int window, int fold, SigmoidArgs sig = SigmoidArgs{0, nullptr, nullptr, 0}) {
+                          int H, int Hkv, float scale, int window, int fold, SigmoidArgs sig = SigmoidArgs{0, nullptr, nullptr, 0, 0}) {
     // the stages of K and V tiles are static LDS (four of 16 KiB per key group with D = 128)
     hipLaunchKernelGGL((attention_prefill_kernel<D, NT, KW, SIG>), grid, dim3(AP_THREADS * KW), 0, stream, (const bf16*)q,
                        q_stride, (bf16*)out, out_stride, (const bf16*)k_pages, (const bf16*)v_pages, block_table,
@@ -691,8 +712,13 @@ static int launch_prefill(dim3 grid, hipStream_t stream, const void* q, long q_s
 extern "C" int mv_attention_prefill(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
                                     const void* v_pages, const int* block_table, int bt_width, int page_size,
                                     const int* positions, const int* cu_seqlens, int n_seqs, int n_units, int n_busy,
-                                    int nt, int kw, int H, int Hkv, int D, float scale, int window, hipStream_t stream) {
+                                    int nt, int kw, int H, int Hkv, int D, float scale, int window, int first,
+                                    const void* gate, long gate_stride, hipStream_t stream) {
     MV_REQUIRE(kw == 1 || kw == 2, "attention_prefill: %d key groups per workgroup (1 or 2)", kw);
+    MV_REQUIRE(first >= 0 && (gate == nullptr || gate_stride >= H), "attention_prefill: bad count of kept first positions or "
+               "gate rows too short");
+    if (window < 0) first = 0;             // without a window every key is seen anyway
+    const SigmoidArgs extra{0, nullptr, (const bf16*)gate, gate_stride, first};
     MV_REQUIRE(H > 0 && Hkv > 0 && H % Hkv == 0, "attention_prefill: %d heads are not a multiple of %d kv heads", H,
                Hkv);
     MV_REQUIRE(D == 64 || D == 128, "attention_prefill: head_dim %d is not served by the MFMA kernel (64 or 128)", D);
@@ -718,7 +744,7 @@ extern "C" int mv_attention_prefill(const void* q, long q_stride, void* out, lon
 #define AP_LAUNCH(DD, NN, KK)                                                                                      \
     rc = launch_prefill<DD, NN, KK>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table,       \
                                     bt_width, page_size, page_shift, positions, cu_seqlens, n_seqs, H, Hkv, scale,  \
-                                    window, fold)
+                                    window, fold, extra)
     if (kw == 2) {
         if (D == 128 && nt == 2) AP_LAUNCH(128, 2, 2);
         else if (D == 128) AP_LAUNCH(128, 1, 2);
@@ -766,7 +792,7 @@ extern "C" int mv_attention_prefill_sigmoid(const void* q, long q_stride, void* 
         cus = 256;
     if (n_busy <= 0 || n_busy > n_units) n_busy = n_units;
     const int fold = (kw == 1 && (long)Hkv * n_busy <= 2L * cus) ? 1 : 0;
-    const SigmoidArgs sig{chunk, bias, (const bf16*)gate, gate_stride};
+    const SigmoidArgs sig{chunk, bias, (const bf16*)gate, gate_stride, 0};
     int rc = 0;
 #define AP_LAUNCH(DD, NN, KK)                                                                                          \
     rc = launch_prefill<DD, NN, KK, true>(grid, stream, q, q_stride, out, out_stride, k_pages, v_pages, block_table,     \

@@ -149,9 +149,11 @@ _OPTIONAL_SIGNATURES = {
     # A, lda, W, bias, C, ldc, c_dtype, M, N, K, gated, partial, P, eps, stream
     "mv_gemm_tile_scaled": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int,
                                     c_int, c_void_p, c_int, c_float, c_void_p]),
+    # q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width, page_size, positions, cu_seqlens, n_seqs, H, Hkv,
+    # D, scale, window, partials, counters, nsplit, max_pages, waves, token_seq, first, gate, gate_stride, stream
     "mv_attention_decode": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int,
-                                    c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+                                    c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_long, c_void_p]),
     # qkv, stride, q_off, k_off, v_off, out, out_stride, k_pages, v_pages, block_table, bt_width, page_size,
     # positions, cu_seqlens, n_seqs, H, Hkv, D, scale, window, q_weight, k_weight, weight_dtype, eps, unit_offset,
     # table, rows, store_kv, partials, counters, nsplit, max_pages, waves, token_seq, stream
@@ -162,9 +164,10 @@ _OPTIONAL_SIGNATURES = {
     # ids, table, table_dtype, resid, n, h, vocab, scale, ids2, table2, out2, h2, rows2, stream
     "mv_embedding_gather": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p,
                                     c_void_p, c_int, c_int, c_void_p]),
+    # ..., positions, cu_seqlens, n_seqs, n_units, n_busy, nt, kw, H, Hkv, D, scale, window, first, gate, gate_stride, stream
     "mv_attention_prefill": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                     c_float, c_int, c_void_p]),
+                                     c_float, c_int, c_int, c_void_p, c_long, c_void_p]),
     "mv_attention_prefill_unit_tokens": (c_int, [c_int, c_int]),
     # as mv_attention_prefill up to window, then chunk, bias, gate, gate_stride, stream
     "mv_attention_prefill_sigmoid": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,

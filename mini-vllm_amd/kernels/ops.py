@@ -1911,8 +1911,6 @@ class Ops:
         """The MFMA kernels, when the step and the sizes allow them."""
         if not self.use_fast_kernels or plan is None or not self.lib.has("mv_attention_decode"):
             return False
-        if first > 0 or gate is not None:
-            return False
         if D not in (64, 128) or page_size % 16 or qs % 8 or os_ % 4 or q.data_ptr() % 16 or out.data_ptr() % 8:
             return False
         group = H // Hkv
@@ -1925,7 +1923,7 @@ class Ops:
                           positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, H, Hkv, D, float(scale), window,
                           _ptr(partials), self._split_counters(n_seqs * Hkv, partials), nsplit,
                           -(-max(1, plan.max_context_len) // page_size), DECODE_ATTENTION_WAVES, token_seq.data_ptr(),
-                          self._stream())
+                          first, _ptr(gate), gs, self._stream())
             return True
         if page_size & (page_size - 1):
             return False
@@ -1936,7 +1934,7 @@ class Ops:
         self.lib.call("mv_attention_prefill", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                       positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, n_units, n_busy, nt, kw, H, Hkv, D,
-                      float(scale), window, self._stream())
+                      float(scale), window, first, _ptr(gate), gs, self._stream())
         return True
 
     # ------------------------------------------------------------------------------------

@@ -633,7 +633,7 @@ def test_attention_decode_one_workgroup_over_more_pages_than_it_stages():
     seq0 = dev(torch.zeros(1, dtype=torch.int32))
     ops.lib.call("mv_attention_decode", qd.data_ptr(), H * D, out.data_ptr(), H * D, kp.data_ptr(), vp.data_ptr(),
                  bt.data_ptr(), pages, ps, pos.data_ptr(), cu.data_ptr(), 1, H, Hkv, D, D ** -0.5, -1, 0, 0, 1, 0, 4,
-                 seq0.data_ptr(), ops._stream())
+                 seq0.data_ptr(), 0, 0, 0, ops._stream())
     torch.cuda.synchronize()
     want = reference_attention(q.double(), k_all, v_all, torch.tensor([ctx - 1]), torch.tensor([0]), H, Hkv, D ** -0.5, None)
     assert rel_err(out.float().cpu().view(1, H, D).numpy(), want.numpy()) <= 2 * OP_TOL[dtype]

@@ -218,9 +218,10 @@ class AttentionCase:
             out[:, hd] = torch.softmax(s, -1) @ k0[:, hd // (H // G)]
         return (out * gate[:, :, None]).reshape(n, H * D)
 
-    def run(self, steps, window, first, scale, drop_pages=False):
+    def run(self, steps, window, first, scale, drop_pages=False, variant=None):
         """Feeds the request in steps of the given sizes; returns [n, H * D]. ``drop_pages``: a page that neither the
-        window nor the kept positions need any more is taken out of the block table (and filled with NaN) before a step."""
+        window nor the kept positions need any more is taken out of the block table (and filled with NaN) before a step.
+        ``variant``: (column tiles a wave, key groups a workgroup) of the MFMA prompt kernel instead of the launch rule's."""
         from minivllm_amd.engine.step import AttentionPlan
         from minivllm_amd.parts.base import Workspace
         H, G, D, page = self.H, self.G, self.D, self.page
@@ -242,7 +243,7 @@ class AttentionCase:
                                         self.v_pages, bt, page, value_from_key=True, extra_columns=self.width - held)
             out = torch.empty(k, H * D, dtype=self.dtype, device=DEV)
             plan = AttentionPlan(decode_only=(k == 1), max_q_len=k, max_context_len=p + k, n_seqs=1, q_lens=[k],
-                                 cu_seqlens=i32([0, k]), workspace=ws)
+                                 cu_seqlens=i32([0, k]), workspace=ws, prefill_variant=variant if k > 1 else None)
             self.ops.attention(packed[:, :H * D], out, self.k_pages, self.v_pages, bt, page, positions, tsq, H, G, D, scale,
                                window - 1, plan=plan, keep_first=first, gate=packed[:, held:held + H])
             rows.append(out)
@@ -288,6 +289,28 @@ def test_one_key_that_stands_out_is_seen_exactly_where_the_mask_says(dtype, sing
         else:
             assert float(hit.abs().max()) < 1.0, f"key {target} should not be seen: {hit.tolist()}"
         close(got.view(1, -1), case.want(window, first, 1.0)[n - 1:n], 3e-5 if dtype == torch.float32 else 2.5e-2, f"key {target}")
+
+
+@pytest.mark.parametrize("nt, kw", [(1, 1), (1, 2), (2, 1), (2, 2)])
+@pytest.mark.parametrize("H, G, window, first", [(4, 2, 36, 13), (3, 1, 50, 33), (2, 2, 20, 40)])
+def test_kept_positions_in_every_variant_of_the_prompt_kernel(nt, kw, H, G, window, first):
+    """Every query points at one kept position, so its output is that key's value wherever it lies. A unit of queries
+    whose first windows still reach the block of the kept positions and whose last ones do not must look at that block
+    for all of them, with four waves and with eight (two groups that take the blocks of keys in turn)."""
+    dtype, D, page, n = torch.bfloat16, 64, 16, 300
+    case = AttentionCase(H, G, D, 0, 1.0, n, page, seed=nt * 10 + kw + window, dtype=dtype, gain=0.3)
+    direction = torch.zeros(D)
+    direction[3] = 1.0
+    target = first - 1
+    case.packed[target, H * D:H * D + G * D] = (6.0 * direction).repeat(G).to(dtype)
+    case.packed[:, :H * D] = (6.0 * direction).repeat(H).to(dtype)
+    case.packed[:, H * D + G * D:H * D + G * D + H] = 8.0
+    want = case.want(window, first, 1.0)
+    for steps in ([n], [5, 128, 64, 3, 100], [61, 2, 237]):
+        got = case.run(steps, window, first, 1.0, drop_pages=True, variant=(nt, kw))
+        hit = got.double().cpu().view(n, H, D)[target:, :, 3]
+        assert float(hit.min()) > 5.0, f"steps {steps}: the kept key is lost at {int((hit.min(1).values < 5.0).nonzero()[0]) + target}"
+        close(got, want, 2.5e-2, f"steps {steps}")
 
 
 # ---------------------------------------------------------------------------------------
