@@ -37,6 +37,11 @@ of the named shape's sizes (``minivllm_amd.config.shapes.bolapel_shape``: the sh
 vocabulary, head counts and number of layers; three delta-rule layers to one attention layer in chunks of
 ``--chunk`` tokens), so that the two designs can be read side by side; the default design and workload are Qwen3's.
 
+``--design zedudra`` does the same for a Zedudra model of the named shape's sizes (``zedudra_shape``: every layer
+attention over a window of ``--window`` positions beside the first ``--keep-first``, every ``--dense-every``-th
+feed-forward dense and the others mixtures of ``--experts`` experts of which a token uses ``--top``); with
+``--dense-every 1`` every feed-forward is dense, which is the model to read beside Qwen3 of the same shape.
+
 Weights are seeded random tensors of the named shape and prompts are seeded uniform token ids
 (there is no network for checkpoints or datasets). The reference publishes no number for this
 metric, so ``vs_baseline`` is null.
@@ -84,6 +89,10 @@ def build_llm(args, shape, layers, max_seqs=None, token_budget=None, num_pages=N
     elif getattr(args, "design", "qwen3") == "dutilix":
         from minivllm_amd.config.shapes import dutilix_shape
         raw = dict(dutilix_shape(args.shape, layers, experts=args.experts, top=args.top), torch_dtype=args.dtype)
+    elif getattr(args, "design", "qwen3") == "zedudra":
+        from minivllm_amd.config.shapes import zedudra_shape
+        raw = dict(zedudra_shape(args.shape, layers, window=args.window, keep_first=args.keep_first, experts=args.experts,
+                                 top=args.top, dense_every=args.dense_every), torch_dtype=args.dtype)
     else:
         raw = dict(shape, architectures=["Qwen3ForCausalLM"], num_hidden_layers=layers,
                    max_position_embeddings=40960, torch_dtype=args.dtype)
@@ -440,6 +449,79 @@ def bench_dutilix(args, llm, cfg, layers, layers_full, item) -> int:
     return 0
 
 
+def zedudra_numbers(llm, cfg, item):
+    """From the loaded model: elements of all tensors; of the matrices every token multiplies with; of all expert
+    matrices and of those a token uses; bytes of convolution state a request reads and writes a step; cache bytes a
+    token takes in each layer with the keys that layer's queries see at most."""
+    from minivllm_amd.models.causal_lm import expected_tensors
+    ex = llm.executor
+    decls = expected_tensors(ex.arch, cfg, ex.plan)
+    params = sum(_numel(d.shape) for d in decls.values())
+    expert = sum(_numel(d.shape) for n, d in decls.items() if ".mlp.e" in n)
+    matrices = sum(_numel(d.shape) for n, d in decls.items() if len(d.shape) == 2 and n != "embed" and ".mlp.e" not in n
+                   and not n.endswith(".canon1"))
+    routers = [(l.mlp.experts, l.mlp.top) for l in cfg.layers if l.mlp is not None and l.mlp.kind == "moe"]
+    per_layer_expert = expert // max(1, len(routers))
+    active = sum(per_layer_expert * min(t, e) // max(e, 1) for e, t in routers)
+    state_bytes = sum(t[0].numel() * t.element_size() for ts in ex.state_tensors.values() for t in ts.values())
+    attn = [(l.mixer.heads, l.mixer.kv_heads, l.mixer.dim, l.mixer.window, l.mixer.keep_first) for l in cfg.layers]
+    return dict(params=params, matrices=matrices, expert=expert, active=active, routers=routers,
+                per_layer_expert=per_layer_expert, state_bytes=state_bytes, attn=attn)
+
+
+def _visible_pairs(T, window, first):
+    """(query, key) pairs of a prompt of T tokens under a window of ``window`` positions beside the first ``first``."""
+    return sum(min(t + 1, window) + max(0, min(first, t + 1 - window)) for t in range(T))
+
+
+def bench_zedudra(args, llm, cfg, layers, layers_full, item) -> int:
+    """The default measurements for a Zedudra model of the named shape; the same fields in the line."""
+    nums = zedudra_numbers(llm, cfg, item)
+    prefill = None
+    if args.only in ("all", "prefill"):
+        prefill_s = measure_prefill(llm, cfg.vocab_size, args.prefill_tokens, repeats=3, seed=args.seed)
+        T = args.prefill_tokens
+        flops = 2 * T * (nums["matrices"] + nums["active"] - cfg.vocab_size * cfg.hidden_size) + 2 * cfg.vocab_size * cfg.hidden_size
+        for H, G, D, window, first in nums["attn"]:
+            flops += 4 * H * D * _visible_pairs(T, window, first)
+        prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+                   "frac": round(flops / prefill_s / PEAK_FLOPS[args.dtype], 4)}
+    tok_s = ms_step = roofline = None
+    ran = regions = 0
+    if args.only in ("all", "decode"):
+        tok_s, ms_step, mean_ctx, ran, regions = measure_decode(llm, cfg.vocab_size, args.batch, args.prompt_len,
+                                                                args.steps, args.warmup, args.seed)
+        # every weight that some request of the step uses once (of a layer's E experts about E (1 - (1 - top/E)^batch)),
+        # each request's convolution inputs read and written, the keys its queries see read twice (as keys and as values)
+        touched = sum(nums["per_layer_expert"] * (1.0 - (1.0 - min(t, e) / e) ** args.batch) for e, t in nums["routers"])
+        seen = sum(2 * G * D * item * min(mean_ctx, window + first) for H, G, D, window, first in nums["attn"])
+        step_bytes = (nums["params"] - nums["expert"] + touched) * item + args.batch * (2 * nums["state_bytes"] + seen)
+        achieved = step_bytes / (ms_step * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(achieved / PEAK_HBM_GBS, 4)}
+    points = {}
+    if not args.no_points and args.only == "all":
+        for b, key in ((1, "decode_b1"), (64, "decode_b64")):
+            n = min(args.steps, 128)
+            points[key] = round(measure_decode(llm, cfg.vocab_size, b, args.prompt_len, n, min(args.warmup, 8),
+                                               args.seed + b)[0], 1)
+    config = {"model": f"zedudra-{args.shape}-shape-random", "layers": layers, "layers_full": layers_full,
+              "hidden": cfg.hidden_size, "vocab": cfg.vocab_size, "window": args.window, "keep_first": args.keep_first,
+              "moe_layers": len(nums["routers"]), "experts": args.experts, "top": args.top, "weights": nums["params"],
+              "weights_a_token_uses": nums["params"] - nums["expert"] + nums["active"], "global_batch": args.batch,
+              "seq_len": args.context, "prompt_len": args.prompt_len, "block_size": args.block_size, "graph": not args.no_graph,
+              "scheduler_steps": args.scheduler_steps, "launch_ahead": bool(llm.config.launch_ahead),
+              "parallelism": "single-gpu"}
+    print(json.dumps({"metric": "decode tok/s (batch %d, %d-token prompts)" % (args.batch, args.prompt_len),
+                      "value": round(tok_s, 1) if tok_s is not None else None, "unit": "tokens/s", "n_gpus": 1,
+                      "steps": ran if ran else args.steps, "warmup": args.warmup,
+                      "ms_per_step": round(ms_step, 4) if ms_step is not None else None, "higher_is_better": True,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                      "data": "synthetic", "config": config, "timed_regions": regions, "prefill": prefill,
+                      "roofline": roofline, "points": points}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -448,7 +530,12 @@ def main() -> int:
     ap.add_argument("--shape", choices=sorted(SHAPES), default="0.6b")
     ap.add_argument("--experts", type=int, default=32, help="--design dutilix: experts of each mixture layer")
     ap.add_argument("--top", type=int, default=4, help="--design dutilix: experts a token uses (each 1/top of the dense width)")
-    ap.add_argument("--design", choices=["qwen3", "bolapel", "dutilix"], default="qwen3",
+    ap.add_argument("--window", type=int, default=1024, help="--design zedudra: positions a query sees behind it (itself among them)")
+    ap.add_argument("--keep-first", type=int, default=64, help="--design zedudra: first positions every query keeps seeing")
+    ap.add_argument("--dense-every", type=int, default=2,
+                    help="--design zedudra: every n-th feed-forward is dense, the others are routed (1: all dense; a number "
+                         "above the layer count: only the first)")
+    ap.add_argument("--design", choices=["qwen3", "bolapel", "dutilix", "zedudra"], default="qwen3",
                     help="'bolapel': the same widths, head counts, vocabulary and number of layers as the named Qwen3 "
                          "shape, as a Bolapel model (three delta-rule layers to one attention layer in chunks of --chunk "
                          "tokens); decode and prefill are measured the same way and the line names the design")
@@ -551,6 +638,8 @@ def main() -> int:
         return bench_bolapel(args, llm, cfg, layers, layers_full, item)
     if args.design == "dutilix":
         return bench_dutilix(args, llm, cfg, layers, layers_full, item)
+    if args.design == "zedudra":
+        return bench_zedudra(args, llm, cfg, layers, layers_full, item)
     nums = model_numbers(shape, layers)
 
     prefill = None

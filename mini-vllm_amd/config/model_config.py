@@ -900,11 +900,22 @@ class ZedudraConfig(ModelConfig):
                     if not (1 <= f.top <= f.experts // f.groups * f.groups_keep):
                         raise ConfigError(f"{lw}: top {f.top} exceeds the experts that can be chosen")
             if l.weights_of is not None:
-                j = l.weights_of
-                if not (0 <= j < i) or self.layers[j].weights_of is not None:
-                    raise ConfigError(f"{lw}: weights_of {j} must name an earlier layer with tensors of its own")
+                j = self.owner_of(i, lw)
                 if (self.layers[j].mixer, self.layers[j].mlp) != (l.mixer, l.mlp):
                     raise ConfigError(f"{lw}: weights_of {j} names a layer with other sizes or constants than this one")
+
+    def owner_of(self, i: int, where: str = "layers") -> int:
+        """The layer whose tensors layer ``i`` uses: itself, or the end of its chain of ``weights_of`` (a layer may
+        name one that itself uses another's; the chain may point backwards or forwards but must end)."""
+        seen = {i}
+        while self.layers[i].weights_of is not None:
+            j = self.layers[i].weights_of
+            if not (0 <= j < len(self.layers)) or j in seen:
+                raise ConfigError(f"{where}: weights_of {j} must name another layer of the model, and the chain must end "
+                                  f"at a layer with tensors of its own")
+            seen.add(j)
+            i = j
+        return i
 
     def to_dict(self) -> Dict[str, Any]:
         layers = []

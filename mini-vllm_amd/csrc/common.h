@@ -101,6 +101,37 @@ struct WeightPtr {
     }
 };
 
+// Eight consecutive elements, read and written 16 bytes (bf16) or 32 bytes (float) at a time.
+template <typename T> struct Vec8;
+template <> struct Vec8<bf16> {
+    static __device__ __forceinline__ void load(const bf16* p, float (&x)[8]) {
+        const uint4 u = *reinterpret_cast<const uint4*>(p);
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            x[2 * e] = __uint_as_float(w[e] << 16);
+            x[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ void store(bf16* p, const float (&x)[8]) {
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            w[e] = f32x2_to_bf16x2_bits(x[2 * e], x[2 * e + 1]);
+        *reinterpret_cast<uint4*>(p) = uint4{w[0], w[1], w[2], w[3]};
+    }
+};
+template <> struct Vec8<float> {
+    static __device__ __forceinline__ void load(const float* p, float (&x)[8]) {
+        const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+        x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+    }
+    static __device__ __forceinline__ void store(float* p, const float (&x)[8]) {
+        *reinterpret_cast<float4*>(p) = float4{x[0], x[1], x[2], x[3]};
+        *reinterpret_cast<float4*>(p + 4) = float4{x[4], x[5], x[6], x[7]};
+    }
+};
+
 // ---------------------------------------------------------------------------------------
 // Reductions
 // ---------------------------------------------------------------------------------------

@@ -63,37 +63,6 @@ extern "C" int mv_embedding_gather(const int* ids, const void* table, int table_
     return mv_check_launch("embedding_gather");
 }
 
-// Eight consecutive elements, read and written 16 bytes (bf16) or 32 bytes (float) at a time.
-template <typename T> struct Vec8;
-template <> struct Vec8<bf16> {
-    static __device__ __forceinline__ void load(const bf16* p, float (&x)[8]) {
-        const uint4 u = *reinterpret_cast<const uint4*>(p);
-        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            x[2 * e] = __uint_as_float(w[e] << 16);
-            x[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
-        }
-    }
-    static __device__ __forceinline__ void store(bf16* p, const float (&x)[8]) {
-        uint32_t w[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            w[e] = f32x2_to_bf16x2_bits(x[2 * e], x[2 * e + 1]);
-        *reinterpret_cast<uint4*>(p) = uint4{w[0], w[1], w[2], w[3]};
-    }
-};
-template <> struct Vec8<float> {
-    static __device__ __forceinline__ void load(const float* p, float (&x)[8]) {
-        const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
-        x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
-    }
-    static __device__ __forceinline__ void store(float* p, const float (&x)[8]) {
-        *reinterpret_cast<float4*>(p) = float4{x[0], x[1], x[2], x[3]};
-        *reinterpret_cast<float4*>(p + 4) = float4{x[4], x[5], x[6], x[7]};
-    }
-};
-
 // ---------------------------------------------------------------------------------------
 // Residual add + RMSNorm.
 //   rows == null : for every row r: v = resid[r] + delta[r]; resid[r] = v; out[r] = norm(v) * w
@@ -905,11 +874,33 @@ __global__ void xielu_kernel(const T* __restrict__ x, long ldx, T* __restrict__ 
     out[r * ldo + c] = from_f<T>(v);
 }
 
+// eight neighbouring columns a thread (cols a multiple of 8, rows 16-byte aligned)
+template <typename T>
+__global__ void xielu_vec_kernel(const T* __restrict__ x, long ldx, T* __restrict__ out, long ldo, int cols8, long total8,
+                                 float a_pos, float a_neg) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total8) return;
+    const long r = i / cols8, c = (i % cols8) * 8;
+    float z[8], v[8];
+    Vec8<T>::load(x + r * ldx + c, z);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = z[e] > 0.f ? fmaf(a_pos * z[e], z[e], 0.5f * z[e]) : fmaf(a_neg, expm1f(z[e]) - z[e], 0.5f * z[e]);
+    Vec8<T>::store(out + r * ldo + c, v);
+}
+
 extern "C" int mv_xielu(const void* x, long ldx, void* out, long ldo, int n, int cols, float a_pos, float a_neg, int dtype,
                         hipStream_t stream) {
     MV_REQUIRE(n >= 0 && cols > 0 && ldx >= cols && ldo >= cols && x && out, "xielu: bad sizes n=%d cols=%d", n, cols);
     const long total = (long)n * cols;
     if (total == 0) return 0;
+    const size_t item = dtype == MV_F32 ? 4 : 2;
+    if (cols % 8 == 0 && (ldx * item) % 16 == 0 && (ldo * item) % 16 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+        const long total8 = total / 8;
+        MV_DISPATCH_T(dtype, "xielu",
+                      hipLaunchKernelGGL(xielu_vec_kernel<T>, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, stream, (const T*)x,
+                                         ldx, (T*)out, ldo, cols / 8, total8, a_pos, a_neg));
+        return mv_check_launch("xielu");
+    }
     MV_DISPATCH_T(dtype, "xielu",
                   hipLaunchKernelGGL(xielu_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (const T*)x,
                                      ldx, (T*)out, ldo, cols, total, a_pos, a_neg));

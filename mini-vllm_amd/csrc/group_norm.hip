@@ -144,9 +144,147 @@ group_norm_add_norm_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, floa
     }
 }
 
+// The same for rows of a multiple of 8 columns whose groups are multiples of 8 too, at most 2048 NC columns,
+// everything 16-byte aligned: a thread keeps NC chunks of eight neighbouring columns in registers from the
+// first load to the last store, and everything it needs from memory (with CONV also the request's kept rows
+// and the taps, at most GN_VEC_TAPS of them, given tap by tap: conv_wt[taps][h]) is asked for before the first
+// sum, so the kernel waits for memory once. A chunk's sum of squares goes to LDS; wave w adds the chunks of
+// groups w, w + 4, ... in a fixed order.
+#define GN_VEC_TAPS 4
+template <typename T, int NC, bool CONV>
+__global__ void __launch_bounds__(GN_THREADS)
+group_norm_add_norm_vec_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, float eps_a, float* __restrict__ resid, WeightPtr wb,
+                               float eps_b, int groups, T* __restrict__ out, int h, int conv_taps, WeightPtr conv_wt,
+                               T* __restrict__ conv_state, const int* __restrict__ token_seq, const int* __restrict__ state_slots) {
+    __shared__ float csum[GN_THREADS * NC];
+    __shared__ float rinv[GN_MAX_GROUPS];
+    const int r = blockIdx.x;
+    const int lane = threadIdx.x % MV_WAVE, wave = threadIdx.x / MV_WAVE;
+    const int nchunks = h / 8, gc = nchunks / groups;          // chunks of a row, of a group
+    const T* yr = y + (size_t)r * ldy;
+    float* res = resid + (size_t)r * h;
+    const WeightPtr wbl = out != nullptr ? wb : wa;
+    const int seq = CONV ? token_seq[r] : 0;
+    T* hist = nullptr;
+    if (CONV && seq >= 0 && conv_taps > 1) hist = conv_state + (size_t)state_slots[seq] * (conv_taps - 1) * h;
+    float v[NC][8], xr[NC][8], fa[NC][8], fb[NC][8];
+    float kept[CONV ? NC : 1][GN_VEC_TAPS - 1][8], wt[CONV ? NC : 1][GN_VEC_TAPS][8];
+    int group_of[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int q = threadIdx.x + GN_THREADS * c;
+        const bool ok = q < nchunks;
+        const int d = ok ? 8 * q : 0;                           // beyond the row's end: the first chunk again, dropped
+        group_of[c] = ok ? q / gc : 0;
+        Vec8<T>::load(yr + d, v[c]);
+        Vec8<float>::load(res + d, xr[c]);
+        wa.at8(d, fa[c]);
+        wbl.at8(d, fb[c]);
+        if constexpr (CONV) {
+#pragma unroll
+            for (int j = 0; j < GN_VEC_TAPS; ++j) {
+                if (j < conv_taps) conv_wt.at8((size_t)j * h + d, wt[c][j]);
+                if (j < GN_VEC_TAPS - 1) {
+                    if (hist != nullptr && j < conv_taps - 1) Vec8<T>::load(hist + (size_t)j * h + d, kept[c][j]);
+                }
+            }
+        }
+        float s = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s = fmaf(v[c][e], v[c][e], s);
+        csum[q] = s;
+    }
+    auto group_scales = [&](float eps) {
+        __syncthreads();
+        for (int g = wave; g < groups; g += GN_WAVES) {
+            float s = 0.f;
+            for (int k = lane; k < gc; k += MV_WAVE) s += csum[g * gc + k];
+            s = wave_sum(s);
+            if (lane == 0) rinv[g] = 1.f / sqrtf(s / (float)(8 * gc) + eps);
+        }
+        __syncthreads();
+    };
+    group_scales(eps_a);
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int q = threadIdx.x + GN_THREADS * c;
+        const float ra = rinv[group_of[c]];
+        float s = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            v[c][e] = xr[c][e] + v[c][e] * ra * fa[c][e];
+            s = fmaf(v[c][e], v[c][e], s);
+        }
+        if (q < nchunks) Vec8<float>::store(res + 8 * q, v[c]);
+        csum[q] = s;
+    }
+    if (out == nullptr) return;
+    group_scales(eps_b);
+    T* o = out + (size_t)r * h;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int q = threadIdx.x + GN_THREADS * c;
+        if (q >= nchunks) continue;
+        const float rb = rinv[group_of[c]];
+        float g8[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) g8[e] = v[c][e] * rb * fb[c][e];
+        if constexpr (!CONV) {
+            Vec8<T>::store(o + 8 * q, g8);
+        } else {
+            float acc[8];
+            if (seq < 0) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+                Vec8<T>::store(o + 8 * q, acc);
+                continue;
+            }
+            // the row as it is stored (rounded to T) is what the taps see and what the request keeps
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                g8[e] = to_f(from_f<T>(g8[e]));
+                acc[e] = g8[e];
+            }
+#pragma unroll
+            for (int j = 0; j < GN_VEC_TAPS - 1; ++j) {
+                if (j < conv_taps - 1) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[e] = fmaf(wt[c][j][e], kept[c][j][e], acc[e]);
+                    if (j > 0) Vec8<T>::store(hist + (size_t)(j - 1) * h + 8 * q, kept[c][j]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < GN_VEC_TAPS; ++j) {
+                if (j == conv_taps - 1) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[e] = fmaf(wt[c][j][e], g8[e], acc[e]);
+                }
+            }
+            if (conv_taps > 1) Vec8<T>::store(hist + (size_t)(conv_taps - 2) * h + 8 * q, g8);
+            Vec8<T>::store(o + 8 * q, acc);
+        }
+    }
+}
+
+template <typename T, bool CONV>
+static void launch_add_norm_vec(int nc, int n, hipStream_t stream, const void* y, long ldy, WeightPtr a, float eps_a, float* resid,
+                                WeightPtr b, float eps_b, int groups, void* out, int h, int conv_taps, WeightPtr cwt,
+                                void* conv_state, const int* token_seq, const int* state_slots) {
+#define GN_LAUNCH(NC)                                                                                                       \
+    hipLaunchKernelGGL((group_norm_add_norm_vec_kernel<T, NC, CONV>), dim3(n), dim3(GN_THREADS), 0, stream, (const T*)y, ldy, a, \
+                       eps_a, resid, b, eps_b, groups, (T*)out, h, conv_taps, cwt, (T*)conv_state, token_seq, state_slots)
+    if (nc == 1) GN_LAUNCH(1);
+    else if (nc == 2) GN_LAUNCH(2);
+    else GN_LAUNCH(4);
+#undef GN_LAUNCH
+}
+
+static bool gn_aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
+
+// conv_w [h][taps]; conv_wt the same taps given tap by tap, [taps][h], or null (the vector kernel needs it)
 extern "C" int mv_group_norm_add_norm(const void* y, long ldy, const void* wa, int wa_dtype, float eps_a, float* resid,
                                       const void* wb, int wb_dtype, float eps_b, int groups, void* out, int n, int h,
-                                      int conv_taps, const void* conv_w, int conv_w_dtype, void* conv_state,
+                                      int conv_taps, const void* conv_w, const void* conv_wt, int conv_w_dtype, void* conv_state,
                                       const int* token_seq, const int* state_slots, int dtype, hipStream_t stream) {
     MV_REQUIRE(n >= 0 && h > 0 && groups >= 1 && groups <= GN_MAX_GROUPS && h % groups == 0 && ldy >= h,
                "group_norm_add_norm: rows of %d columns do not form %d equal groups (at most %d)", h, groups, GN_MAX_GROUPS);
@@ -158,6 +296,23 @@ extern "C" int mv_group_norm_add_norm(const void* y, long ldy, const void* wa, i
     MV_REQUIRE((size_t)h * sizeof(float) <= GN_MAX_ROW_BYTES, "group_norm_add_norm: rows of %d columns exceed the %d that fit LDS", h, (int)(GN_MAX_ROW_BYTES / 4));
     if (n == 0) return 0;
     WeightPtr a{wa, wa_dtype}, b{wb, wb_dtype}, cw{conv_w, conv_w_dtype};
+    const size_t item = dtype == MV_F32 ? 4 : 2;
+    if (h % 8 == 0 && (h / groups) % 8 == 0 && h <= 2048 * 4 && (ldy * item) % 16 == 0 && gn_aligned16(y) && gn_aligned16(resid)
+        && gn_aligned16(wa) && (out == nullptr || (gn_aligned16(out) && gn_aligned16(wb)))
+        && (conv_taps == 0 || (conv_taps <= GN_VEC_TAPS && conv_wt != nullptr && gn_aligned16(conv_wt) && gn_aligned16(conv_state)))) {
+        const int nc = h <= 2048 ? 1 : h <= 4096 ? 2 : 4;
+        const WeightPtr cwt{conv_wt, conv_w_dtype};
+        if (conv_taps > 0) {
+            MV_DISPATCH_T(dtype, "group_norm_add_norm",
+                          (launch_add_norm_vec<T, true>(nc, n, stream, y, ldy, a, eps_a, resid, b, eps_b, groups, out, h, conv_taps,
+                                                        cwt, conv_state, token_seq, state_slots)));
+        } else {
+            MV_DISPATCH_T(dtype, "group_norm_add_norm",
+                          (launch_add_norm_vec<T, false>(nc, n, stream, y, ldy, a, eps_a, resid, b, eps_b, groups, out, h, 0, cwt,
+                                                         nullptr, nullptr, nullptr)));
+        }
+        return mv_check_launch("group_norm_add_norm");
+    }
     MV_DISPATCH_T(dtype, "group_norm_add_norm",
                   hipLaunchKernelGGL(group_norm_add_norm_kernel<T>, dim3(n), dim3(GN_THREADS), (size_t)h * sizeof(float), stream,
                                      (const T*)y, ldy, a, eps_a, resid, b, eps_b, groups, (T*)out, h, conv_taps, cw,

@@ -232,7 +232,7 @@ extern "C" int mv_scale_f32(float* x, long ld, int rows, int cols, float factor,
 //                 and pairs without an expert are left out. Within an expert the order of the pairs is
 //                 whatever the counters gave; no result depends on it (a row's products read only its own row).
 //   moe_gate_up   per tile and 128 columns: act[pair] = weight[pair] * silu(x W_gate^T) * (x W_up^T), the rows of x
-//                 gathered through `sorted`, rounded once
+//                 gathered through `sorted`, rounded once (with a `limit` > 0 the clamped pair of moe_swiglu_scale)
 //   moe_down      per tile and 128 columns: out[pair] = act[pair] W_down^T as floats
 //   moe_combine   y[token] = sum over its places (in order) of out[pair] + (identity weights) * x[token]
 //
@@ -295,7 +295,7 @@ __global__ void __launch_bounds__(256)
 moe_expert_product_kernel(const bf16* __restrict__ a, long lda, int a_by_token, const bf16* __restrict__ w, long ldw, int E, int N,
                           int K, const int* __restrict__ sorted, const int* __restrict__ tile_expert,
                           const int* __restrict__ tile_row0, const int* __restrict__ tile_rows, const float* __restrict__ weights,
-                          int top, bf16* __restrict__ act, float* __restrict__ out) {
+                          int top, bf16* __restrict__ act, float* __restrict__ out, float limit, float slope) {
     const int tile = blockIdx.x;
     const int e = tile_expert[tile];
     if (e < 0) return;
@@ -354,7 +354,14 @@ moe_expert_product_kernel(const bf16* __restrict__ a, long lda, int a_by_token, 
             if (col >= N) continue;
             if (GATED) {
                 const float g = acc0[s][idx], u = acc1[s][idx];
-                act[(size_t)p * N + col] = from_f<bf16>(wt * (g / (1.f + expf(-g))) * u);
+                float v;
+                if (limit > 0.f) {          // the clamped pair, as in moe_swiglu_scale
+                    const float gc = fminf(g, limit), uc = fminf(fmaxf(u, -limit), limit);
+                    v = wt * (gc / (1.f + expf(-slope * gc))) * (uc + 1.f);
+                } else {
+                    v = wt * (g / (1.f + expf(-g))) * u;
+                }
+                act[(size_t)p * N + col] = from_f<bf16>(v);
             } else {
                 out[(size_t)p * N + col] = acc0[s][idx];
             }
@@ -385,8 +392,9 @@ extern "C" long mv_moe_grouped_ints(int n, int top, int n_real) { return (long)n
 // returns 2 (nothing done) for sizes it does not serve
 extern "C" int mv_moe_grouped(const void* x, long ldx, int n, int hidden, const void* w_gate_up, const void* w_down, int n_real,
                               int identity, int F, const int* ids, const float* weights, int top, const float* dense,
-                              int ld_dense, int* ints, void* act, float* out, void* y, long ldy, hipStream_t stream) {
-    MV_REQUIRE(n >= 0 && hidden > 0 && n_real > 0 && F > 0 && top > 0 && identity >= 0, "moe_grouped: bad sizes");
+                              int ld_dense, int* ints, void* act, float* out, void* y, long ldy, float limit, float slope,
+                              hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && hidden > 0 && n_real > 0 && F > 0 && top > 0 && identity >= 0 && limit >= 0.f, "moe_grouped: bad sizes");
     if (hidden % 32 || F % 32 || ldx % 8 || ((uintptr_t)x % 16) || ((uintptr_t)w_gate_up % 16) || ((uintptr_t)w_down % 16)
         || ((uintptr_t)act % 16) || n_real > MR_MAX_E)
         return 2;
@@ -404,11 +412,11 @@ extern "C" int mv_moe_grouped(const void* x, long ldx, int n, int hidden, const 
     if (mv_check_launch("moe_sort")) return 1;
     hipLaunchKernelGGL(moe_expert_product_kernel<true>, dim3(max_tiles, (F + MG_COLS - 1) / MG_COLS), dim3(256), 0, stream, (const bf16*)x, ldx,
                        1, (const bf16*)w_gate_up, (long)hidden, n_real, F, hidden, sorted, tile_expert, tile_row0, tile_rows,
-                       weights, top, (bf16*)act, (float*)nullptr);
+                       weights, top, (bf16*)act, (float*)nullptr, limit, slope);
     if (mv_check_launch("moe_gate_up")) return 1;
     hipLaunchKernelGGL(moe_expert_product_kernel<false>, dim3(max_tiles, (hidden + MG_COLS - 1) / MG_COLS), dim3(256), 0, stream,
                        (const bf16*)act, (long)F, 0, (const bf16*)w_down, (long)n_real * F, n_real, hidden, F, sorted, tile_expert,
-                       tile_row0, tile_rows, weights, top, (bf16*)nullptr, out);
+                       tile_row0, tile_rows, weights, top, (bf16*)nullptr, out, 0.f, 0.f);
     if (mv_check_launch("moe_down")) return 1;
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n), dim3(256), 0, stream, out, ids, top, n_real, (const bf16*)x, ldx, dense,
                        ld_dense, identity, (bf16*)y, ldy, hidden);

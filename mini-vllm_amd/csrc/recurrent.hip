@@ -774,8 +774,44 @@ input_conv_kernel(const T* __restrict__ h, long ldh, T* __restrict__ out, long l
     }
 }
 
-// h, ldh, out, ldo: [n][C] rows; w [C][taps]; conv_state [slots][taps-1][C] in the activation type (may be null with one tap)
-extern "C" int mv_input_conv(const void* h, long ldh, void* out, long ldo, const void* w, int weight_dtype, int taps,
+// The same for channels in chunks of eight (C a multiple of 8, rows 16-byte aligned), with the taps given tap by
+// tap, wt[taps][C]: a thread takes eight neighbouring channels of one row, 16 bytes a load. The same sum in the
+// same order as above.
+template <typename T>
+__global__ void __launch_bounds__(256)
+input_conv_vec_kernel(const T* __restrict__ h, long ldh, T* __restrict__ out, long ldo, WeightPtr wt, int taps,
+                      const T* __restrict__ conv_state, const int* __restrict__ token_seq, const int* __restrict__ cu_seqlens,
+                      const int* __restrict__ state_slots, int C, int n) {
+    const int per_row = C / 8;
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long)n * per_row) return;
+    const int t = (int)(idx / per_row), c = (int)(idx % per_row) * 8;
+    const int seq = token_seq[t];
+    T* o = out + (size_t)t * ldo + c;
+    float acc[8];
+    if (seq < 0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+        Vec8<T>::store(o, acc);
+        return;
+    }
+    const int first = cu_seqlens[seq];
+    const T* hist = taps > 1 ? conv_state + (size_t)state_slots[seq] * (taps - 1) * C : nullptr;
+    Vec8<T>::load(h + (size_t)t * ldh + c, acc);
+    for (int j = 0; j < taps; ++j) {
+        const int r = t - (taps - 1) + j;
+        float x[8], w[8];
+        Vec8<T>::load(r >= first ? h + (size_t)r * ldh + c : hist + (size_t)(taps - 1 + (r - first)) * C + c, x);
+        wt.at8((size_t)j * C + c, w);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = fmaf(w[e], x[e], acc[e]);
+    }
+    Vec8<T>::store(o, acc);
+}
+
+// h, ldh, out, ldo: [n][C] rows; w [C][taps] (wt: the same tap by tap, [taps][C], or null); conv_state [slots][taps-1][C] in
+// the activation type (may be null with one tap)
+extern "C" int mv_input_conv(const void* h, long ldh, void* out, long ldo, const void* w, const void* wt, int weight_dtype, int taps,
                              void* conv_state, const int* token_seq, const int* cu_seqlens, const int* state_slots, int n,
                              int n_seqs, int C, int dtype, hipStream_t stream) {
     MV_REQUIRE(n >= 0 && n_seqs >= 0 && C > 0 && ldh >= C && ldo >= C, "input_conv: bad sizes n=%d C=%d", n, C);
@@ -786,9 +822,20 @@ extern "C" int mv_input_conv(const void* h, long ldh, void* out, long ldo, const
     MV_REQUIRE((C + 255) / 256 <= 65535, "input_conv: too many channels");
     if (n == 0) return 0;
     WeightPtr wp{w, weight_dtype};
-    MV_DISPATCH_T(dtype, "input_conv",
-                  hipLaunchKernelGGL(input_conv_kernel<T>, dim3(n), dim3(256), 0, stream, (const T*)h, ldh, (T*)out, ldo, wp, taps,
-                                     (const T*)conv_state, token_seq, cu_seqlens, state_slots, C));
+    const size_t item = dtype == MV_F32 ? 4 : 2;
+    const auto aligned = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
+    if (wt != nullptr && C % 8 == 0 && (ldh * item) % 16 == 0 && (ldo * item) % 16 == 0 && aligned(h) && aligned(out) && aligned(wt)
+        && aligned(conv_state) && (long)n * (C / 8) / 256 + 1 < 0x7fffffffL) {
+        const WeightPtr wtp{wt, weight_dtype};
+        const unsigned blocks = (unsigned)(((long)n * (C / 8) + 255) / 256);
+        MV_DISPATCH_T(dtype, "input_conv",
+                      hipLaunchKernelGGL(input_conv_vec_kernel<T>, dim3(blocks), dim3(256), 0, stream, (const T*)h, ldh, (T*)out, ldo,
+                                         wtp, taps, (const T*)conv_state, token_seq, cu_seqlens, state_slots, C, n));
+    } else {
+        MV_DISPATCH_T(dtype, "input_conv",
+                      hipLaunchKernelGGL(input_conv_kernel<T>, dim3(n), dim3(256), 0, stream, (const T*)h, ldh, (T*)out, ldo, wp, taps,
+                                         (const T*)conv_state, token_seq, cu_seqlens, state_slots, C));
+    }
     if (mv_check_launch("input_conv")) return 1;
     if (taps > 1 && n_seqs > 0) {
         MV_DISPATCH_T(dtype, "conv_state",

@@ -450,7 +450,8 @@ class Executor:
             max_context_len=max((s.start + len(s.tokens) for s in seqs), default=0),
             n_seqs=facts["Sp"], q_lens=list(facts["q_lens"]) + [0] * (facts["Sp"] - facts["S"]),
             cu_seqlens=ctx.cu_seqlens, workspace=self.rt.workspace,
-            kv_tokens=sum(s.start + len(s.tokens) for s in seqs),
+            kv_tokens=sum(s.start + len(s.tokens) for s in seqs), starts=[s.start for s in seqs],
+            step_q_lens=[len(s.tokens) for s in seqs],
             attention_pairs=sum(len(s.tokens) * s.start + len(s.tokens) * (len(s.tokens) + 1) // 2 for s in seqs))
         for call in range(len(self.plan.calls)):
             g = self.group_of_call.get(call)

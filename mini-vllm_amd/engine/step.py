@@ -74,6 +74,10 @@ class AttentionPlan:
     # number of (query, visible key) pairs without windows
     kv_tokens: int = 0
     attention_pairs: int = 0
+    # for measurement: the position of each sequence's first token of the step and its number of tokens, on the
+    # host (a recording for a size class clears ``q_lens``; these stay those of the step that was recorded)
+    starts: Sequence[int] = ()
+    step_q_lens: Sequence[int] = ()
 
     def units(self, unit_tokens: int) -> int:
         """Runs of up to ``unit_tokens`` consecutive tokens of one sequence in the step: counted from

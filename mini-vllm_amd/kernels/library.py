@@ -51,13 +51,13 @@ _SIGNATURES = {
     # resid, x, ldx, delta, weight, weight_dtype, eps, groups, out, ldo, rows, n_out, h, dtype, stream
     "mv_group_norm_rows": (c_int, [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_long,
                                    c_void_p, c_int, c_int, c_int, c_void_p]),
-    # y, ldy, wa, wa_dtype, eps_a, resid, wb, wb_dtype, eps_b, groups, out, n, h, conv_taps, conv_w, conv_w_dtype, conv_state,
-    # token_seq, state_slots, dtype, stream
+    # y, ldy, wa, wa_dtype, eps_a, resid, wb, wb_dtype, eps_b, groups, out, n, h, conv_taps, conv_w, conv_wt, conv_w_dtype,
+    # conv_state, token_seq, state_slots, dtype, stream
     "mv_group_norm_add_norm": (c_int, [c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_float, c_int,
-                                       c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
-                                       c_void_p]),
-    # h, ldh, out, ldo, w, weight_dtype, taps, conv_state, token_seq, cu_seqlens, state_slots, n, n_seqs, C, dtype, stream
-    "mv_input_conv": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                       c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                                       c_int, c_void_p]),
+    # h, ldh, out, ldo, w, wt, weight_dtype, taps, conv_state, token_seq, cu_seqlens, state_slots, n, n_seqs, C, dtype, stream
+    "mv_input_conv": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                               c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     # x, ldx, out, ldo, n, cols, a_pos, a_neg, dtype, stream
     "mv_xielu": (c_int, [c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_float, c_float, c_int, c_void_p]),
@@ -105,9 +105,10 @@ _OPTIONAL_SIGNATURES = {
     "mv_attention_latent_mfma": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                          c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p]),
     "mv_moe_grouped_ints": (c_long, [c_int, c_int, c_int]),
-    # x, ldx, n, hidden, w_gate_up, w_down, n_real, identity, F, ids, weights, top, dense, ld_dense, ints, act, out, y, ldy, stream
+    # x, ldx, n, hidden, w_gate_up, w_down, n_real, identity, F, ids, weights, top, dense, ld_dense, ints, act, out, y, ldy,
+    # limit, slope, stream
     "mv_moe_grouped": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int,
-                               c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p]),
+                               c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_float, c_float, c_void_p]),
     "mv_gemm_skinny": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int,
                                c_int, c_int, c_int, c_void_p]),
     "mv_gemm_skinny_swiglu": (c_int, [c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_void_p]),

@@ -476,10 +476,12 @@ class Ops:
                       token_seq.data_ptr(), cu_seqlens.data_ptr(), state_slots.data_ptr(), n, w, self.code, self._stream())
 
     def input_conv(self, h: torch.Tensor, taps: torch.Tensor, state: Optional[torch.Tensor], token_seq: torch.Tensor,
-                   cu_seqlens: torch.Tensor, state_slots: torch.Tensor, n_seqs: int, out: torch.Tensor) -> None:
+                   cu_seqlens: torch.Tensor, state_slots: torch.Tensor, n_seqs: int, out: torch.Tensor,
+                   taps_t: Optional[torch.Tensor] = None) -> None:
         """out[t] = h[t] + sum_j taps[:, j] * h[t - T + 1 + j] along each request's rows (T = taps.shape[1], the last tap
         multiplies h[t]); the rows in front of a request's first row of the step are state[slot] [T - 1, w], which then
-        takes the request's last T - 1 rows. h, out [n, w]; taps [w, T]; state [slots, T - 1, w] (None with one tap)."""
+        takes the request's last T - 1 rows. h, out [n, w]; taps [w, T]; state [slots, T - 1, w] (None with one tap).
+        ``taps_t`` [T, w]: the same taps tap by tap, which lets the kernel take eight channels a thread."""
         self._act(h, "convolution input"); self._act(out, "convolution output"); _dev(taps, "convolution taps")
         n, w = h.shape
         if out.shape != h.shape or h.stride(1) != 1 or out.stride(1) != 1 or out.data_ptr() == h.data_ptr():
@@ -493,9 +495,19 @@ class Ops:
                 raise KernelLibraryError(f"input_conv: state {tuple(state.shape)} does not hold {T - 1} rows of {w}")
         self._ints(n, token_seq=(token_seq, n), cu_seqlens=(cu_seqlens, n_seqs + 1), state_slots=(state_slots, n_seqs))
         self._note("mv_input_conv", self._size(h, out) + (T - 1) * n_seqs * w * h.element_size() * 2, 2 * T * n * w)
+        taps_t = self._taps_by_tap(taps, taps_t, "input_conv")
         self.lib.call("mv_input_conv", h.data_ptr(), h.stride(0) if n > 1 else w, out.data_ptr(), out.stride(0) if n > 1 else w,
-                      taps.data_ptr(), _weight_code(taps, "convolution taps"), T, _ptr(state) if T > 1 else 0,
+                      taps.data_ptr(), _ptr(taps_t), _weight_code(taps, "convolution taps"), T, _ptr(state) if T > 1 else 0,
                       token_seq.data_ptr(), cu_seqlens.data_ptr(), state_slots.data_ptr(), n, n_seqs, w, self.code, self._stream())
+
+    @staticmethod
+    def _taps_by_tap(taps: torch.Tensor, taps_t: Optional[torch.Tensor], what: str) -> Optional[torch.Tensor]:
+        if taps_t is None:
+            return None
+        _dev(taps_t, "convolution taps, tap by tap")
+        if tuple(taps_t.shape) != (taps.shape[1], taps.shape[0]) or taps_t.dtype != taps.dtype or not taps_t.is_contiguous():
+            raise KernelLibraryError(f"{what}: taps given tap by tap {tuple(taps_t.shape)} do not mirror the taps {tuple(taps.shape)}")
+        return taps_t
 
     def group_norm(self, weight: torch.Tensor, eps: float, groups: int, out: torch.Tensor, resid: Optional[torch.Tensor] = None,
                    x: Optional[torch.Tensor] = None, delta: Optional[torch.Tensor] = None,
@@ -540,8 +552,9 @@ class Ops:
         """resid += gnorm(y) * w (``norm_y`` = (weight, eps)); with ``norm_next`` of the same form, out = gnorm(resid) * w'.
         Both norms work in ``groups`` runs of columns; the sum stays float32 in between.
 
-        ``conv`` = (taps [h, T], state [slots, T - 1, h] or None, token_seq, state_slots), for steps in which every request
-        brings one token: ``out`` gets the rows after the input convolution that ``input_conv`` would apply to them."""
+        ``conv`` = (taps [h, T], state [slots, T - 1, h] or None, token_seq, state_slots[, taps tap by tap [T, h]]), for steps
+        in which every request brings one token: ``out`` gets the rows after the input convolution that ``input_conv`` would
+        apply to them."""
         self._act(y, "sublayer output"); _dev(resid, "residual")
         n, h = resid.shape
         if resid.dtype != torch.float32 or not resid.is_contiguous() or tuple(y.shape) != (n, h) or y.stride(1) != 1:
@@ -560,10 +573,10 @@ class Ops:
             wb_code = _weight_code(wb, "norm weight")
             if wb.numel() != h or not wb.is_contiguous() or tuple(out.shape) != (n, h) or not out.is_contiguous():
                 raise KernelLibraryError("group_norm_add_norm: the second norm's weight or output does not fit")
-        taps = state = tsq = slots = None
+        taps = taps_t = state = tsq = slots = None
         T, taps_code = 0, DTYPE_F32
         if conv is not None:
-            taps, state, tsq, slots = conv
+            taps, state, tsq, slots = conv[:4]
             if out is None:
                 raise KernelLibraryError("group_norm_add_norm: a convolution needs the second norm and its output")
             _dev(taps, "convolution taps")
@@ -576,10 +589,11 @@ class Ops:
                 if tuple(state.shape[1:]) != (T - 1, h) or not state.is_contiguous():
                     raise KernelLibraryError(f"group_norm_add_norm: state {tuple(state.shape)} does not hold {T - 1} rows of {h}")
             self._ints(n, token_seq=(tsq, n), state_slots=(slots, 1))
+            taps_t = self._taps_by_tap(taps, conv[4] if len(conv) > 4 else None, "group_norm_add_norm")
         self._note("mv_group_norm_add_norm", self._size(y, out) + 2 * self._size(resid), 8 * n * h)
         self.lib.call("mv_group_norm_add_norm", y.data_ptr(), y.stride(0) if n > 1 else h, wa.data_ptr(),
                       _weight_code(wa, "norm weight"), float(eps_a), resid.data_ptr(), _ptr(wb), wb_code, float(eps_b), int(groups),
-                      _ptr(out), n, h, T, _ptr(taps), taps_code, _ptr(state) if T > 1 else 0, _ptr(tsq), _ptr(slots),
+                      _ptr(out), n, h, T, _ptr(taps), _ptr(taps_t), taps_code, _ptr(state) if T > 1 else 0, _ptr(tsq), _ptr(slots),
                       self.code, self._stream())
 
     def xielu(self, x: torch.Tensor, a_pos: float, a_neg: float, out: torch.Tensor) -> None:
@@ -1066,9 +1080,10 @@ class Ops:
 
     def moe_grouped(self, x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, experts: int, identity: int, ff: int,
                     ids: torch.Tensor, weights: torch.Tensor, dense: torch.Tensor, ints: torch.Tensor, act: torch.Tensor,
-                    out: torch.Tensor, y: torch.Tensor) -> bool:
+                    out: torch.Tensor, y: torch.Tensor, limit: float = 0.0, slope: float = 1.0) -> bool:
         """The experts' products over the chosen (token, expert) pairs only (bfloat16): y[t] = sum over t's chosen experts
-        of weight * down_e(silu(gate_e x) * up_e x) + (its identity experts' weights) * x[t]. ``w_gate_up`` is
+        of weight * down_e(silu(gate_e x) * up_e x) + (its identity experts' weights) * x[t]; with ``limit`` > 0 the pair
+        is the clamped one, g = min(gate, limit), u = clamp(up, -limit, limit), g * sigmoid(slope * g) * (u + 1). ``w_gate_up`` is
         [2 * experts * ff, hidden] (all gate blocks, then all up blocks), ``w_down`` [hidden, experts * ff]; ids / weights
         [n, top] and dense [n, experts + identity] as ``moe_route`` leaves them; ``ints`` (int32), ``act`` [n * top, ff]
         and ``out`` float32 [n * top, hidden] are scratch. False when the sizes are not served (nothing was done)."""
@@ -1092,7 +1107,7 @@ class Ops:
         if not self.lib.offer("mv_moe_grouped", x.data_ptr(), x.stride(0) if n > 1 else hidden, n, hidden, w_gate_up.data_ptr(),
                               w_down.data_ptr(), experts, identity, ff, ids.data_ptr(), weights.data_ptr(), top, dense.data_ptr(),
                               dense.stride(0) if n > 1 else dense.shape[1], ints.data_ptr(), act.data_ptr(), out.data_ptr(),
-                              y.data_ptr(), y.stride(0) if n > 1 else hidden, self._stream()):
+                              y.data_ptr(), y.stride(0) if n > 1 else hidden, float(limit), float(slope), self._stream()):
             return False
         used = min(experts, n * top)
         self._note("mv_moe_grouped", self._size(x, y) + used * 3 * ff * hidden * 2 + self._size(act, out) * 2,
@@ -1177,6 +1192,24 @@ class Ops:
         priced = copy.copy(plan)
         priced.kv_tokens = min(plan.kv_tokens, seqs * chunk + tokens)
         priced.attention_pairs = min(plan.attention_pairs, tokens * chunk)
+        return priced
+
+    @staticmethod
+    def _window_priced(plan, window: int, first: int):
+        """For the ledger: under a window (``window`` positions behind the query, beside the first ``first``) a
+        request's queries read the keys from the window of its first query on and the kept ones, and a query at
+        position p makes min(p, window) + 1 pairs and one for each kept position that the window has let go of."""
+        if plan is None or window < 0 or not plan.starts or len(plan.starts) != len(plan.step_q_lens):
+            return plan
+        import copy
+        keys = pairs = 0
+        for start, ql in zip(plan.starts, plan.step_q_lens):
+            lo = max(0, start - window)
+            keys += start + ql - lo + min(first, lo)
+            for p in range(start, start + ql):
+                pairs += min(p, window) + 1 + max(0, min(first, p - window))
+        priced = copy.copy(plan)
+        priced.kv_tokens, priced.attention_pairs = keys, pairs
         return priced
 
     def attention_sigmoid(self, q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
@@ -1792,14 +1825,15 @@ class Ops:
                     pass
             raise
 
-    def _decode_split(self, plan, n_seqs: int, H: int, Hkv: int, D: int):
+    def _decode_split(self, plan, n_seqs: int, H: int, Hkv: int, D: int, context: Optional[int] = None):
         """Over how many workgroups a decode step deals a sequence's keys out, and the work area for
         their partial results: (nsplit, partials). The keys go round in groups of 128 (a block of 32
         to each of a workgroup's four waves), so a split beyond the number of such groups in the
         planned context would only add workgroups that end at once. The count is a property of the
         plan (a captured graph keeps it): about one workgroup in flight for every compute unit (measured on MI355X with 8 kv heads at contexts of 1,100: 512 and 1,024
         workgroups are 5 and 18 % slower at batch 8; batch 64 is fastest without a split)."""
-        ctx = max(1, plan.max_context_len)
+        # (``context``: the keys a query reads at most, where a window makes that fewer than the planned context)
+        ctx = max(1, plan.max_context_len if context is None else min(context, plan.max_context_len))
         forced = getattr(plan, "decode_splits", None)
         nsplit = forced if forced else max(1, min(self.compute_units // max(1, n_seqs * Hkv), -(-ctx // 128), 64))
         partials = None
@@ -1915,9 +1949,12 @@ class Ops:
             return False
         group = H // Hkv
         n_seqs = plan.n_seqs
+        priced = self._window_priced(plan, window, first) if self.ledger is not None else plan
         if plan.decode_only and group <= 16:
-            nsplit, partials = self._decode_split(plan, n_seqs, H, Hkv, D)
-            self._note_attention("mv_attention_decode", plan, q.shape[0], H, Hkv, D, 2, splits=nsplit)
+            # under a window a query reads the window, the kept positions and what the blocks of 32 add at both ends
+            nsplit, partials = self._decode_split(plan, n_seqs, H, Hkv, D,
+                                                  context=None if window < 0 else window + 1 + first + 64)
+            self._note_attention("mv_attention_decode", priced, q.shape[0], H, Hkv, D, 2, splits=nsplit)
             self._decode_launch("mv_attention_decode", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                           v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                           positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, H, Hkv, D, float(scale), window,
@@ -1930,7 +1967,7 @@ class Ops:
         nt, kw, n_units, n_busy = self._prefill_variant(plan, group, Hkv)
         if nt == 0:
             return False
-        self._note_attention("mv_attention_prefill", plan, q.shape[0], H, Hkv, D, 2)
+        self._note_attention("mv_attention_prefill", priced, q.shape[0], H, Hkv, D, 2)
         self.lib.call("mv_attention_prefill", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
                       positions.data_ptr(), plan.cu_seqlens.data_ptr(), n_seqs, n_units, n_busy, nt, kw, H, Hkv, D,

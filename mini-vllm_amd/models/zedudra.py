@@ -37,10 +37,11 @@ def zedudra_plan(config: ZedudraConfig) -> ModelPlan:
     norm = GroupRMSNormSpec(size=hid, eps=config.norm_eps, groups=config.norm_groups)
     block = SandwichBlockSpec(hidden_size=hid, input_conv_taps=config.conv_taps)
     layers, calls = [], []
-    index_of: Dict[int, int] = {}          # config layer with tensors of its own -> layer of the plan
+    # config layer with tensors of its own -> layer of the plan
+    index_of: Dict[int, int] = {i: k for k, i in enumerate(_owners(config))}
     for i, l in enumerate(config.layers):
         if l.weights_of is not None:
-            calls.append(Call(layer=index_of[l.weights_of]))
+            calls.append(Call(layer=index_of[config.owner_of(i)]))
             continue
         m = l.mixer
         rope = RotarySpec(rotary_dim=m.rot_dims, theta=m.rot_base, interleaved=True) if m.rot_dims else None
@@ -58,7 +59,7 @@ def zedudra_plan(config: ZedudraConfig) -> ModelPlan:
                                     keep_groups=f.groups_keep, correction=False, scoring="sigmoid", group_worth="top2",
                                     normalize=False, activation="clamped", limit=f.limit, gate_slope=GATE_SLOPE)
         slots = SandwichBlock.slots_for(ffn is not None)
-        index_of[i] = len(layers)
+        assert index_of[i] == len(layers)
         layers.append(LayerPlan(block=block, mixer=mixer, ffn=ffn, norms=tuple((s, norm) for s in slots)))
         calls.append(Call(layer=index_of[i]))
     plan = ModelPlan(hidden_size=hid, vocab_size=config.vocab_size, max_positions=config.max_position_embeddings,

@@ -136,6 +136,8 @@ class SandwichBlock(Block):
         self.canon = (tensors or {}).get("canon")
         if spec.input_conv_taps > 0 and (self.canon is None or rt is None):
             raise ValueError("a block with an input convolution needs its 'canon' tensor and the runtime")
+        # the same taps tap by tap, [taps, width]: the kernels then read eight channels' weights of a tap in one load
+        self.canon_t = self.canon.t().contiguous() if self.canon is not None else None
         if spec.input_conv_taps > 0 and spec.token_shift:
             raise ValueError("a block shapes its mixer's input by a token shift or by a convolution, not both")
 
@@ -146,7 +148,7 @@ class SandwichBlock(Block):
         # the rows pass through the shift first: no product takes the norm over; a block in front may
         # apply this block's shift together with its norm (``TokenShiftEntry``)
         if self.canon is not None:
-            return InputConvEntry(self.canon)
+            return InputConvEntry(self.canon, self.canon_t)
         return TokenShiftEntry(self.shift) if self.shift is not None else None
 
     def _conv_state(self, ctx, call: int):
@@ -164,7 +166,7 @@ class SandwichBlock(Block):
         elif self.canon is not None and not already:
             mixed = self.rt.workspace.get("conv.out", tuple(h.shape), h.dtype)
             self.rt.ops.input_conv(h, self.canon, self._conv_state(ctx, call), ctx.token_seq, ctx.cu_seqlens,
-                                   ctx.state_slots, ctx.n_seqs, mixed)
+                                   ctx.state_slots, ctx.n_seqs, mixed, taps_t=self.canon_t)
             h = mixed
         y = self.mixer.forward(h, ctx, call)
         last = self.ffn is None
@@ -223,7 +225,7 @@ class SandwichBlock(Block):
         if rows is not None and isinstance(next_part, InputConvEntry) and plan is not None and plan.decode_only:
             taps = next_part.taps
             state = ctx.state(call + 1, "conv.last") if taps.shape[1] > 1 else None    # the block that runs next is call + 1
-            conv = (taps, state, ctx.token_seq, ctx.state_slots)
+            conv = (taps, state, ctx.token_seq, ctx.state_slots, next_part.taps_t)
         self.rt.ops.group_norm_add_norm(y, (wa, eps_a), stream.resid, second, rows, groups, conv=conv)
         stream.delta = None
         if rows is None:
@@ -237,8 +239,8 @@ class InputConvEntry:
     """What a sandwich block with an input convolution offers the block in front of it: the taps, so that
     its rows can leave that block's last kernel with the convolution applied."""
 
-    def __init__(self, taps: torch.Tensor):
-        self.taps = taps
+    def __init__(self, taps: torch.Tensor, taps_t: Optional[torch.Tensor] = None):
+        self.taps, self.taps_t = taps, taps_t
 
 
 class TokenShiftEntry:

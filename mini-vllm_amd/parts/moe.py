@@ -111,7 +111,7 @@ class RoutedExperts(FeedForward):
     def wants_grouped(self, n: int) -> bool:
         """Whether a step of n rows computes the chosen pairs only (where the kernels take the sizes)."""
         spec = self.spec
-        return (spec.grouped and spec.activation == "swiglu" and n * spec.top < spec.grouped_max_rows * spec.num_experts
+        return (spec.grouped and n * spec.top < spec.grouped_max_rows * spec.num_experts
                 and spec.expert_size * spec.hidden_size >= spec.grouped_min_weight)
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
@@ -132,7 +132,8 @@ class RoutedExperts(FeedForward):
             need = int(ops.lib.dll.mv_moe_grouped_ints(n, spec.top, n_e)) if ops.lib.has("mv_moe_grouped") else 0
             if need and ops.moe_grouped(x, self.w_gate_up, self.w_down, n_e, spec.identity_experts, F, ids, weights, dense,
                                         ws.get("moe.ints", (need,), torch.int32), ws.get("moe.pair_act", (n * spec.top, F), rt.dtype),
-                                        ws.get("moe.pair_out", (n * spec.top, spec.hidden_size), torch.float32), y):
+                                        ws.get("moe.pair_out", (n * spec.top, spec.hidden_size), torch.float32), y,
+                                        limit=spec.limit if spec.activation == "clamped" else 0.0, slope=spec.gate_slope):
                 return y
         if n_e:
             gu = ws.get("moe.gate_up", (n, 2 * n_e * F), rt.dtype)

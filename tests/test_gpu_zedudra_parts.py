@@ -72,8 +72,12 @@ def test_group_norm_rows(dtype, h, groups):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("h, groups, taps", [(64, 4, 3), (50, 5, 2), (256, 1, 4), (32, 16, 1), (48, 2, 0)])
+@pytest.mark.parametrize("h, groups, taps", [(64, 4, 3), (50, 5, 2), (256, 1, 4), (32, 16, 1), (48, 2, 0), (4096, 4, 4), (8192, 2, 3),
+                                             (1024, 128, 2), (2056, 1, 1), (3072, 3, 5), (640, 80, 3), (8200, 1, 2)])
 def test_norm_add_norm_in_groups_and_the_convolution_riding_along(dtype, h, groups, taps):
+    """Rows the vector kernel takes (a multiple of eight columns in groups of a multiple of eight, up to 8,192, at most
+    four taps given tap by tap) and rows it leaves to the general one; both against the plain norm, and the convolution
+    that rides along against the separate kernel bit for bit."""
     ops = ops_for(dtype)
     g = torch.Generator().manual_seed(h)
     n = 5
@@ -96,17 +100,32 @@ def test_norm_add_norm_in_groups_and_the_convolution_riding_along(dtype, h, grou
     cw = (0.5 * torch.randn(h, taps, generator=g)).to(torch.bfloat16).to(DEV)
     state = torch.randn(4, max(taps - 1, 1), h, generator=g).to(dtype).to(DEV)[:, :taps - 1].contiguous() if taps > 1 else None
     tsq, cu, slots = i32([0, -1, 1, 2, -1]), i32([0, 1, 2, 3]), i32([3, 0, 2])
-    s1 = state.clone() if state is not None else None
-    r3, out3 = resid.clone(), torch.empty(n, h, dtype=dtype, device=DEV)
-    ops.group_norm_add_norm(y, (wa, 1e-5), r3, (wb, 2e-6), out3, groups, conv=(cw, s1, tsq, slots))
-    # the same through the separate kernels on the three real rows
+    cwt = cw.t().contiguous()
     real = [0, 2, 3]
-    s2 = state.clone() if state is not None else None
-    mixed = torch.empty(3, h, dtype=dtype, device=DEV)
-    ops.input_conv(out[real].contiguous(), cw, s2, i32([0, 1, 2]), cu, slots, 3, mixed)
-    assert torch.equal(out3[real], mixed) and float(out3[[1, 4]].abs().max()) == 0
-    if state is not None:
-        assert torch.equal(s1, s2) and torch.equal(s1[1], state[1])      # slot 1 belongs to nobody in the step
+    for by_tap in (False, True):
+        s1 = state.clone() if state is not None else None
+        r3, out3 = resid.clone(), torch.empty(n, h, dtype=dtype, device=DEV)
+        ops.group_norm_add_norm(y, (wa, 1e-5), r3, (wb, 2e-6), out3, groups,
+                                conv=(cw, s1, tsq, slots, cwt) if by_tap else (cw, s1, tsq, slots))
+        close(r3, v, 1e-6, "the residual after the add, with the convolution riding along")
+        # the same through the separate kernels on the three real rows
+        s2 = state.clone() if state is not None else None
+        mixed = torch.empty(3, h, dtype=dtype, device=DEV)
+        ops.input_conv(out[real].contiguous(), cw, s2, i32([0, 1, 2]), cu, slots, 3, mixed, taps_t=cwt if by_tap else None)
+        # (taps not given tap by tap go through the general kernel, whose norm sums in another order than the vector
+        # kernel that made ``out``: equal within rounding there, bit for bit otherwise)
+        exact = by_tap and taps <= 4          # the vector kernel takes up to four taps
+        if exact:
+            assert torch.equal(out3[real], mixed)
+        else:
+            close(out3[real], mixed, TOL[dtype], "the convolution riding along, general kernel")
+        assert float(out3[[1, 4]].abs().max()) == 0
+        if state is not None:
+            if exact:
+                assert torch.equal(s1, s2)
+            else:
+                close(s1, s2, TOL[dtype], "the kept rows, general kernel")
+            assert torch.equal(s1[1], state[1])      # slot 1 belongs to nobody in the step
 
 
 # ---------------------------------------------------------------------------------------
@@ -117,8 +136,9 @@ def conv_reference(h, taps, before):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width, taps", [(64, 3), (50, 2), (256, 4), (30, 1), (40, 7)])
-def test_input_convolution_mixed_step(dtype, width, taps):
+@pytest.mark.parametrize("by_tap", [False, True])
+@pytest.mark.parametrize("width, taps", [(64, 3), (50, 2), (256, 4), (30, 1), (40, 7), (4096, 4), (1032, 16)])
+def test_input_convolution_mixed_step(dtype, width, taps, by_tap):
     """Three requests in one step (a long portion, a portion shorter than the taps reach back, a single token) in slots
     2, 0, 3 with non-zero kept rows, padding rows and a padding sequence; then a second step on what the first left."""
     ops = ops_for(dtype)
@@ -131,7 +151,7 @@ def test_input_convolution_mixed_step(dtype, width, taps):
         h = torch.randn(n + 2, width, generator=g).to(dtype).to(DEV)
         tsq, cu, slots = step_ints(q_lens, [2, 0, 3], pad_rows=2, pad_seqs=1)
         out = torch.full((n + 2, width), 5.0, dtype=dtype, device=DEV)
-        ops.input_conv(h, cw, state, tsq, cu, slots, 4, out)
+        ops.input_conv(h, cw, state, tsq, cu, slots, 4, out, taps_t=cw.t().contiguous() if by_tap else None)
         p = 0
         for s, ql in enumerate(q_lens):
             slot = [2, 0, 3][s]
@@ -330,6 +350,15 @@ def test_xielu(dtype):
     wide[:, :70] = x
     ops.xielu(wide[:, :70], float(plain.softplus(p)), 0.5 + float(plain.softplus(q)), wide[:, :70])      # in place, strided
     assert torch.equal(wide[:, :70], out)
+    # rows of a multiple of eight columns go eight columns a thread; the same numbers as one column a thread
+    x8 = (3 * torch.randn(33, 264, generator=g)).to(dtype).to(DEV)
+    x8[1, 5:9] = torch.tensor([0.0, -0.0, 1e-3, -1e-3]).to(dtype)
+    out8 = torch.empty_like(x8)
+    ops.xielu(x8, float(plain.softplus(p)), 0.5 + float(plain.softplus(q)), out8)
+    close(out8, plain.xielu(x8.double().cpu(), p, q), TOL[dtype], "xielu, eight columns a thread")
+    odd = torch.empty(33, 263, dtype=dtype, device=DEV)
+    ops.xielu(x8[:, :263], float(plain.softplus(p)), 0.5 + float(plain.softplus(q)), odd)
+    assert torch.equal(odd, out8[:, :263])
 
 
 @pytest.mark.parametrize("E, groups, keep, top", [(16, 4, 2, 3), (8, 4, 2, 4), (6, 1, 1, 2), (5, 5, 3, 2), (3, 1, 1, 3),
@@ -382,6 +411,43 @@ def test_routed_clamped_experts_against_the_plain_mixture(dtype, hid, F, E, grou
     f = {"expert": {"ff": F, "limit": limit}, "router": {"experts": E, "top": top, "groups": {"count": groups, "keep": keep}}}
     want = plain.moe_ff(x.double(), names, "mlp.", f)
     close(got, want, 3e-5 if dtype == torch.float32 else 3e-2, "mixture")
+
+
+@pytest.mark.parametrize("n, hid, F, E, groups, keep, top, limit", [(5, 64, 32, 8, 4, 2, 3, 1.5), (70, 96, 64, 6, 1, 1, 2, 0.7),
+                                                                    (1, 128, 32, 16, 2, 1, 4, 2.0)])
+def test_clamped_experts_over_the_chosen_pairs_only(n, hid, F, E, groups, keep, top, limit):
+    """The path that computes only the chosen (token, expert) pairs (bfloat16, steps of few rows against large experts)
+    with the clamped pair in its first product: against the plain mixture, and the kernels it ran are the grouped ones."""
+    from minivllm_amd.parts.base import Runtime, Workspace
+    from minivllm_amd.parts.moe import RoutedExperts, RoutedExpertsSpec
+    dtype = torch.bfloat16
+    ops = ops_for(dtype)
+    g = torch.Generator().manual_seed(n + E)
+    w = {"router": 3 * torch.randn(E, hid, generator=g) / hid ** 0.5}
+    for e in range(E):
+        w[f"gate.{e}"] = 2 * torch.randn(F, hid, generator=g) / hid ** 0.5
+        w[f"up.{e}"] = 2 * torch.randn(F, hid, generator=g) / hid ** 0.5
+        w[f"down.{e}"] = torch.randn(hid, F, generator=g) / F ** 0.5
+    w = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    spec = RoutedExpertsSpec(hidden_size=hid, expert_size=F, num_experts=E, top=top, groups=groups, keep_groups=keep,
+                             scoring="sigmoid", group_worth="top2", normalize=False, activation="clamped", limit=limit,
+                             grouped=True, grouped_max_rows=1e9, grouped_min_weight=0)
+    rt = Runtime(device=torch.device(DEV), dtype=dtype, ops=ops, workspace=Workspace(torch.device(DEV)), max_positions=64)
+    part = RoutedExperts(spec, {k: v.to(DEV) for k, v in w.items()}, rt)
+    x = torch.randn(n, hid, generator=g).to(dtype)
+    ledger, ops.ledger = ops.ledger, []
+    try:
+        got = part.forward(x.to(DEV), None).clone()
+        seen = [line[0] for line in ops.ledger]
+    finally:
+        ops.ledger = ledger
+    assert "mv_moe_grouped" in seen and "mv_moe_swiglu_scale" not in seen, seen
+    names = {"mlp.router": w["router"].double()}
+    for e in range(E):
+        names.update({f"mlp.e{e}.gate": w[f"gate.{e}"].double(), f"mlp.e{e}.up": w[f"up.{e}"].double(),
+                      f"mlp.e{e}.down": w[f"down.{e}"].double()})
+    f = {"expert": {"ff": F, "limit": limit}, "router": {"experts": E, "top": top, "groups": {"count": groups, "keep": keep}}}
+    close(got, plain.moe_ff(x.double(), names, "mlp.", f), 3e-2, "mixture over the chosen pairs")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -276,3 +276,29 @@ def test_a_request_past_a_thousand_tokens(cases, dtype):
     got = trace_tools.collect(steps, runner_for(case, dtype, steps).run_step)
     assert len(got) == len(rows) + 2 + 40
     judge([rel_err(row, want[pos]) for (_, pos), row in got.items()], tol, dtype, "1,100 tokens")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prompt_beside_a_request_past_a_thousand_tokens(cases, dtype):
+    """While one request decodes past 1,024 tokens (steps with so long a context walk the keys with two wave groups
+    a workgroup), another's prompt comes in beside it in portions whose queries straddle the place where the window
+    lets go of the kept first positions' block."""
+    case = cases[("C", "sharp")]
+    long, short = random_tokens(case.cfg, 1060, seed=78), random_tokens(case.cfg, 200, seed=79)
+    want = {"long": plain_logits(case.cfg, case.weights, long), "short": plain_logits(case.cfg, case.weights, short)}
+    steps = [{"step": 0, "entries": [{"id": "long", "tokens": long[:1030], "want": [1029]}], "end": []}]
+    at, cuts = 0, [3, 125, 2, 64, 6]
+    for i in range(30):
+        entries = [{"id": "long", "tokens": [long[1030 + i]], "want": [0]}]
+        if i < len(cuts):
+            entries.append({"id": "short", "tokens": short[at:at + cuts[i]], "want": list(range(cuts[i]))})
+            at += cuts[i]
+        steps.append({"step": 1 + i, "entries": entries, "end": ["long", "short"] if i == 29 else []})
+    assert at == len(short)
+    got = trace_tools.collect(steps, runner_for(case, dtype, steps).run_step)
+    assert len(got) == 1 + 30 + len(short)
+    rows = [(rid, pos) for rid, pos in got]
+    tol = TOL_F32 if dtype == "float32" else bf16_tolerance(max(
+        rel_err(plain_logits_bf16(case.cfg, case.weights, short)[p], want["short"][p]) for p in range(len(short))))
+    judge([rel_err(got[(rid, pos)], want[rid][pos]) for rid, pos in rows], max(tol, case.tol(dtype)), dtype,
+          "a prompt beside a long request")

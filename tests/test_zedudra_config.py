@@ -54,8 +54,10 @@ def test_defaults_and_optional_keys():
     (lambda c: c["layers"][1]["mlp"]["router"].update(top=5), "top"),
     (lambda c: c["layers"][1]["mlp"]["expert"].update(limit=0.0), "limit"),
     (lambda c: c["layers"][0]["mlp"].update(kind="sparse"), "not supported"),
-    (lambda c: c["layers"][2].update(weights_of=3), "weights_of"),
-    (lambda c: c["layers"][3].update(weights_of=2), "weights_of"),
+    (lambda c: c["layers"][2].update(weights_of=2), "weights_of"),
+    (lambda c: c["layers"][3].update(weights_of=5), "weights_of"),
+    (lambda c: (c["layers"][2].update(weights_of=3), c["layers"][3].update(weights_of=2)), "weights_of"),
+    (lambda c: c["layers"][3].update(weights_of=0), "other sizes"),
     (lambda c: c["layers"][2]["mixer"]["mask"].update(size=13), "other sizes"),
     (lambda c: c["norm"].update(groups=3), "norm groups"),
     (lambda c: c["canon"].update(taps=40), "canon.taps"),
@@ -67,6 +69,24 @@ def test_config_errors(edit, message):
     edit(cfg)
     with pytest.raises(ConfigError, match=message):
         load(cfg)
+
+
+def test_a_layer_may_name_a_later_one_or_one_that_names_another():
+    from minivllm_amd.models.causal_lm import expected_tensors
+    arch, want = load(ZED_A)
+    chained = copy.deepcopy(ZED_A)
+    chained["layers"][3]["weights_of"] = 2                      # 3 -> 2 -> 1
+    _, cfg = load(chained)
+    assert [c.layer for c in arch.plan(cfg).calls] == [0, 1, 1, 1, 2]
+    assert set(expected_tensors(arch, cfg)) == set(expected_tensors(arch, want))
+    ahead = copy.deepcopy(ZED_A)
+    ahead["layers"][1]["weights_of"] = 3                        # the tensors are the fourth entry's: l3.*
+    ahead["layers"][2]["weights_of"] = 3
+    del ahead["layers"][3]["weights_of"]
+    _, cfg = load(ahead)
+    assert [c.layer for c in arch.plan(cfg).calls] == [0, 1, 1, 1, 2]
+    names = set(expected_tensors(arch, cfg))
+    assert "l3.mix.q" in names and not any(n.startswith(("l1.", "l2.")) for n in names)
 
 
 def test_plan_parts_calls_and_memory():
