@@ -70,10 +70,10 @@ KERNELS_OF: Dict[str, Tuple[str, Optional[str], int]] = {
     "mv_moe_swiglu_scale": (r"\bmoe_swiglu_scale_kernel", None, 1),
     "mv_moe_identity_add": (r"\bmoe_identity_add_kernel", None, 1),
     "mv_scale_f32": (r"\bscale_f32_kernel", None, 1),
-    "mv_input_conv": (r"\binput_conv_kernel", r"\bconv_state_kernel", 2),
+    "mv_input_conv": (r"\binput_conv(_vec)?_kernel", r"\bconv_state_kernel", 2),
     "mv_group_norm_rows": (r"\bgroup_norm_rows_kernel", None, 1),
-    "mv_group_norm_add_norm": (r"\bgroup_norm_add_norm_kernel", None, 1),
-    "mv_xielu": (r"\bxielu_kernel", None, 1),
+    "mv_group_norm_add_norm": (r"\bgroup_norm_add_norm(_vec)?_kernel", None, 1),
+    "mv_xielu": (r"\bxielu(_vec)?_kernel", None, 1),
     "mv_moe_grouped": (r"\bmoe_sort_kernel", r"\bmoe_(expert_product|combine)_kernel", 4),
 }
 _OURS = re.compile("|".join(f"(?:{p})" for spec in KERNELS_OF.values() for p in spec[:2] if p))
