@@ -489,7 +489,7 @@ qk_norm_rope_store_vec(long block, T* __restrict__ qkv, long row_stride, int q_o
                        const int* __restrict__ block_table, int bt_width, int page_size,
                        T* __restrict__ k_pages, T* __restrict__ v_pages, int n, int H, int Hkv,
                        WeightPtr qw, WeightPtr kw, int has_norm, float eps, int unit_offset,
-                       const float* __restrict__ table, int store_kv) {
+                       const float* __restrict__ table, int store_kv, int rot_dim = 8 * L, int interleaved = 0) {
     // A group of L lanes takes HP heads of one token in turn: the token's angles (twice a head's
     // bytes when the table is float) and the norm weights are read once for all of them.
     constexpr int D = 8 * L;
@@ -503,7 +503,18 @@ qk_norm_rope_store_vec(long block, T* __restrict__ qkv, long row_stride, int q_o
     const bool active = tok < n && seq >= 0;
     const int pos = active ? positions[tok] : 0;
     float c[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, sn[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (table != nullptr) {
+    if (table != nullptr && interleaved) {
+        // neighbouring pairs (2p, 2p + 1) over the first rot_dim channels: a lane's eight elements are four whole pairs,
+        // p = 4 j + m; a pair beyond the rotated part turns by the angle 0
+        const float* cs = table + (size_t)pos * rot_dim;
+        const int half = rot_dim / 2;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            const int p = 4 * j + m;
+            c[m] = p < half ? cs[p] : 1.f;
+            sn[m] = p < half ? cs[half + p] : 0.f;
+        }
+    } else if (table != nullptr) {
         const float* cs = table + (size_t)pos * D + 8 * (j % (L / 2));
         const float4 c0 = *reinterpret_cast<const float4*>(cs), c1 = *reinterpret_cast<const float4*>(cs + 4);
         const float4 s0 = *reinterpret_cast<const float4*>(cs + D / 2);
@@ -550,7 +561,14 @@ qk_norm_rope_store_vec(long block, T* __restrict__ qkv, long row_stride, int q_o
 #pragma unroll
                 for (int e = 0; e < 8; ++e) x[e] = x[e] * rinv * (kind == 0 ? wq[e] : wk[e]);
             }
-            if (table != nullptr) {
+            if (table != nullptr && interleaved) {
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    const float a = x[2 * m], b = x[2 * m + 1];
+                    x[2 * m] = a * c[m] - b * sn[m];
+                    x[2 * m + 1] = b * c[m] + a * sn[m];
+                }
+            } else if (table != nullptr) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float other = __shfl_xor(x[e], L / 2, MV_WAVE);
@@ -583,10 +601,10 @@ qk_norm_rope_store_vec_kernel(T* __restrict__ qkv, long row_stride, int q_off, i
                               const int* __restrict__ block_table, int bt_width, int page_size,
                               T* __restrict__ k_pages, T* __restrict__ v_pages, int n, int H, int Hkv,
                               WeightPtr qw, WeightPtr kw, int has_norm, float eps, int unit_offset,
-                              const float* __restrict__ table, int store_kv) {
+                              const float* __restrict__ table, int store_kv, int rot_dim, int interleaved) {
     qk_norm_rope_store_vec<T, L, HP>(blockIdx.x, qkv, row_stride, q_off, k_off, v_off, positions, token_seq, block_table,
                                      bt_width, page_size, k_pages, v_pages, n, H, Hkv, qw, kw, has_norm, eps, unit_offset,
-                                 table, store_kv);
+                                 table, store_kv, rot_dim, interleaved);
 }
 
 // Value rows of 16 consecutive tokens of the step and one kv head into the transposed value pages
@@ -674,11 +692,12 @@ qkv_prompt_vec_kernel(T* __restrict__ qkv, long row_stride, int q_off, int k_off
                       const int* __restrict__ positions, const int* __restrict__ token_seq,
                       const int* __restrict__ block_table, int bt_width, int page_size, T* __restrict__ k_pages,
                       T* __restrict__ v_pages, int n, int H, int Hkv, WeightPtr qw, WeightPtr kw, int has_norm,
-                      float eps, int unit_offset, const float* __restrict__ table, int qk_blocks) {
+                      float eps, int unit_offset, const float* __restrict__ table, int qk_blocks, int rot_dim,
+                      int interleaved) {
     if ((int)blockIdx.x < qk_blocks) {
         qk_norm_rope_store_vec<T, L, HP>(blockIdx.x, qkv, row_stride, q_off, k_off, v_off, positions, token_seq,
                                      block_table, bt_width, page_size, k_pages, v_pages, n, H, Hkv, qw, kw, has_norm,
-                                     eps, unit_offset, table, 2);
+                                     eps, unit_offset, table, 2, rot_dim, interleaved);
         return;
     }
     __shared__ float tile[16][8 * L + 1];
@@ -692,7 +711,7 @@ template <typename T>
 static bool launch_qk_vec(T* qkv, long row_stride, int q_off, int k_off, int v_off, const int* positions,
                           const int* token_seq, const int* block_table, int bt_width, int page_size, T* k_pages,
                           T* v_pages, int n, int H, int Hkv, int D, WeightPtr qw, WeightPtr kw, int has_norm, float eps,
-                          int unit_offset, const float* table, int store_kv, hipStream_t stream) {
+                          int unit_offset, const float* table, int store_kv, int rot_dim, int interleaved, hipStream_t stream) {
     const bool v_tiles = store_kv == 3;     // keys per head here, values tile by tile in the same launch
     if (v_tiles) store_kv = 2;
     const int heads = H + (store_kv == 1 ? 2 * Hkv : (store_kv == 2 ? Hkv : 0));
@@ -707,12 +726,13 @@ static bool launch_qk_vec(T* qkv, long row_stride, int q_off, int k_off, int v_o
     if (v_tiles)                                                                                                   \
         hipLaunchKernelGGL((qkv_prompt_vec_kernel<T, LL, PP>), grid, dim3(256), 0, stream, qkv, row_stride, q_off, \
                            k_off, v_off, positions, token_seq, block_table, bt_width, page_size, k_pages, v_pages, \
-                           n, H, Hkv, qw, kw, has_norm, eps, unit_offset, table, (int)qk_blocks);                  \
+                           n, H, Hkv, qw, kw, has_norm, eps, unit_offset, table, (int)qk_blocks, rot_dim,         \
+                           interleaved);                                                                           \
     else                                                                                                           \
         hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<T, LL, PP>), grid, dim3(256), 0, stream, qkv,            \
                            row_stride, q_off, k_off, v_off, positions, token_seq, block_table, bt_width,           \
                            page_size, k_pages, v_pages, n, H, Hkv, qw, kw, has_norm, eps, unit_offset, table,      \
-                           store_kv)
+                           store_kv, rot_dim, interleaved)
 #define QK_VEC(LL)                                                                                                 \
     do {                                                                                                           \
         if (hp == 4) { QK_VEC_HP(LL, 4); } else { QK_VEC_HP(LL, 1); }                                              \
@@ -756,19 +776,21 @@ extern "C" int mv_qk_norm_rope_store(void* qkv, long row_stride, int q_off, int 
     if (n == 0) return 0;
     const int heads = H + (store_kv == 1 ? 2 * Hkv : (store_kv >= 2 ? Hkv : 0));
     WeightPtr qw{q_weight, weight_dtype}, kw{k_weight, weight_dtype};
-    // the vector kernel: rotation over the whole head in half-split pairs, everything 16-byte aligned
+    // the vector kernel: rotation over the whole head in half-split pairs, or over any even number of leading channels
+    // in neighbouring pairs; everything 16-byte aligned
     const size_t esz = dtype == MV_F32 ? 4 : 2;
     const bool aligned = ((uintptr_t)qkv % 16) == 0 && (row_stride * esz) % 16 == 0 && (q_off * esz) % 16 == 0 &&
                          (k_off * esz) % 16 == 0 && (v_off * esz) % 16 == 0 && ((uintptr_t)k_pages % 16) == 0 &&
                          ((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0 &&
                          ((uintptr_t)table % 16) == 0;
-    if (aligned && (D == 64 || D == 128 || D == 256 || D == 512) && (table == nullptr || (rot_dim == D && !interleaved)) &&
+    if (aligned && (D == 64 || D == 128 || D == 256 || D == 512) && (table == nullptr || (rot_dim == D && !interleaved) || interleaved) &&
         (long)n * heads * (D / 8) < (1L << 31)) {
         bool took = false;
         MV_DISPATCH_T(dtype, "qk_norm_rope_store",
                       took = launch_qk_vec<T>((T*)qkv, row_stride, q_off, k_off, v_off, positions, token_seq,
                                               block_table, bt_width, page_size, (T*)k_pages, (T*)v_pages, n, H, Hkv, D,
-                                              qw, kw, has_norm, eps, unit_offset, table, store_kv, stream));
+                                              qw, kw, has_norm, eps, unit_offset, table, store_kv, rot_dim,
+                                              interleaved ? 1 : 0, stream));
         if (took) return mv_check_launch("qk_norm_rope_store");
     }
     dim3 grid(n, (heads + 3) / 4);

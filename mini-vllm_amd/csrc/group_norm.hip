@@ -164,9 +164,6 @@ group_norm_add_norm_vec_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, 
     const T* yr = y + (size_t)r * ldy;
     float* res = resid + (size_t)r * h;
     const WeightPtr wbl = out != nullptr ? wb : wa;
-    const int seq = CONV ? token_seq[r] : 0;
-    T* hist = nullptr;
-    if (CONV && seq >= 0 && conv_taps > 1) hist = conv_state + (size_t)state_slots[seq] * (conv_taps - 1) * h;
     float v[NC][8], xr[NC][8], fa[NC][8], fb[NC][8];
     float kept[CONV ? NC : 1][GN_VEC_TAPS - 1][8], wt[CONV ? NC : 1][GN_VEC_TAPS][8];
     int group_of[NC];
@@ -182,12 +179,23 @@ group_norm_add_norm_vec_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, 
         wbl.at8(d, fb[c]);
         if constexpr (CONV) {
 #pragma unroll
-            for (int j = 0; j < GN_VEC_TAPS; ++j) {
+            for (int j = 0; j < GN_VEC_TAPS; ++j)
                 if (j < conv_taps) conv_wt.at8((size_t)j * h + d, wt[c][j]);
-                if (j < GN_VEC_TAPS - 1) {
-                    if (hist != nullptr && j < conv_taps - 1) Vec8<T>::load(hist + (size_t)j * h + d, kept[c][j]);
-                }
-            }
+        }
+    }
+    // the request's kept rows hang on two loads in a row (the row's request, its slot): asked for behind everything
+    // that does not, so that those loads are on their way meanwhile
+    const int seq = CONV ? token_seq[r] : 0;
+    T* hist = nullptr;
+    if (CONV && seq >= 0 && conv_taps > 1) hist = conv_state + (size_t)state_slots[seq] * (conv_taps - 1) * h;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int q = threadIdx.x + GN_THREADS * c;
+        if constexpr (CONV) {
+            const int d = q < nchunks ? 8 * q : 0;
+#pragma unroll
+            for (int j = 0; j < GN_VEC_TAPS - 1; ++j)
+                if (hist != nullptr && j < conv_taps - 1) Vec8<T>::load(hist + (size_t)j * h + d, kept[c][j]);
         }
         float s = 0.f;
 #pragma unroll
