@@ -178,9 +178,10 @@ group_norm_add_norm_vec_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, 
         wa.at8(d, fa[c]);
         wbl.at8(d, fb[c]);
         if constexpr (CONV) {
+            // (every load is issued whatever the number of taps, a tap beyond the last reads the last again and is
+            // dropped: a load under a condition is a branch with a wait of its own)
 #pragma unroll
-            for (int j = 0; j < GN_VEC_TAPS; ++j)
-                if (j < conv_taps) conv_wt.at8((size_t)j * h + d, wt[c][j]);
+            for (int j = 0; j < GN_VEC_TAPS; ++j) conv_wt.at8((size_t)(j < conv_taps ? j : conv_taps - 1) * h + d, wt[c][j]);
         }
     }
     // the request's kept rows hang on two loads in a row (the row's request, its slot): asked for behind everything
@@ -188,6 +189,8 @@ group_norm_add_norm_vec_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, 
     const int seq = CONV ? token_seq[r] : 0;
     T* hist = nullptr;
     if (CONV && seq >= 0 && conv_taps > 1) hist = conv_state + (size_t)state_slots[seq] * (conv_taps - 1) * h;
+    const T* kept_rows = hist != nullptr ? hist : yr;          // (no kept rows: some row that is there, dropped)
+    const int last_kept = hist != nullptr ? conv_taps - 2 : 0;
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
         const int q = threadIdx.x + GN_THREADS * c;
@@ -195,7 +198,7 @@ group_norm_add_norm_vec_kernel(const T* __restrict__ y, long ldy, WeightPtr wa, 
             const int d = q < nchunks ? 8 * q : 0;
 #pragma unroll
             for (int j = 0; j < GN_VEC_TAPS - 1; ++j)
-                if (hist != nullptr && j < conv_taps - 1) Vec8<T>::load(hist + (size_t)j * h + d, kept[c][j]);
+                Vec8<T>::load(kept_rows + (size_t)(j < last_kept ? j : last_kept) * h + d, kept[c][j]);
         }
         float s = 0.f;
 #pragma unroll

@@ -65,7 +65,7 @@ ZED_B = {"architecture": "Zedudra", "vocab": 77, "width": 50, "norm": {"eps": 3e
 ZED_C = {"architecture": "Zedudra", "vocab": 512, "width": 256, "norm": {"eps": 1e-6, "groups": 1}, "canon": {"taps": 4},
          "embedding": {"scale": 16.0},
          "layers": [attn(4, 1, 64, 40, 17, 32, 1000000.0, 0.125, dense(512)),
-                    attn(2, 2, 128, 100, 64, 64, 50000.0, 0.09, moe(128, 2.0, 8, 2, groups=4, keep=2)),
+                    attn(2, 2, 128, 100, 64, 64, 40000.0, 0.09, moe(128, 2.0, 8, 2, groups=4, keep=2)),
                     attn(8, 2, 64, 33, 16, 64, 10000.0, 0.125, moe(64, 1.0, 4, 1, groups=2, keep=1))]}
 # D: one head, one tap (no convolution state), no rotation, every expert chosen, more kept positions than the window is
 # long, a window of one position (a query sees itself and the kept ones), as many norm groups as make pairs of columns
