@@ -167,3 +167,42 @@ def with_layers(cfg: Dict, layers: List[Dict]) -> Dict:
     c = copy.deepcopy(cfg)
     c["layers"] = copy.deepcopy(layers)
     return c
+
+
+def _divisors(n: int) -> List[int]:
+    return [d for d in range(1, n + 1) if n % d == 0]
+
+
+def random_config(rng, dense_only: bool = False) -> Dict:
+    """A configuration drawn at random: width, norm groups, taps, two to six layers that each draw their own head
+    counts, head size, window, kept positions, rotated channels and feed-forward, some of them second calls of an earlier
+    layer. ``dense_only``: heads of 64 or 128 and no mixtures (bfloat16 then stays close to the plain model: no router's
+    near tie can fall the other way)."""
+    width = int(rng.choice([96, 128, 160, 192, 256, 320, 384]))
+    groups = int(rng.choice([g for g in _divisors(width) if g <= 16]))
+    owners, layers = [], []
+    for i in range(int(rng.integers(2, 7))):
+        if owners and rng.random() < 0.35:
+            layers.append(again(layers, int(rng.choice(owners))))
+            continue
+        dim = int(rng.choice([64, 128] if dense_only else [16, 32, 48, 64, 96, 128]))
+        heads = int(rng.choice([1, 2, 3, 4, 6, 8, 12]))
+        rot = min(dim, int(rng.choice([0, 2, 8, 16, dim // 2, dim])))
+        kind = rng.choice(["dense", "dense", "none"] if dense_only else ["dense", "moe", "moe", "none"])
+        if kind == "dense":
+            mlp = dense(int(rng.choice([64, 96, 200, 256, 512])))
+        elif kind == "moe":
+            E = int(rng.choice([4, 6, 8, 12, 16, 32]))
+            g = int(rng.choice(_divisors(E)))
+            keep = int(rng.integers(1, g + 1))
+            mlp = moe(int(rng.choice([32, 64, 96, 128])), float(rng.choice([0.5, 1.0, 2.0, 7.0])), E,
+                      int(rng.integers(1, min(8, E // g * keep) + 1)), groups=g, keep=keep)
+        else:
+            mlp = None
+        owners.append(i)
+        layers.append(attn(heads, int(rng.choice(_divisors(heads))), dim, int(rng.integers(1, 90)),
+                           int(rng.choice([0, 1, 4, 16, 23, 33, 64])), rot - rot % 2, float(rng.choice([100.0, 10000.0, 1e6])),
+                           float(rng.choice([dim ** -0.5, 0.11, 0.2])), mlp))
+    return {"architecture": "Zedudra", "vocab": int(rng.integers(100, 1300)), "width": width,
+            "norm": {"eps": float(rng.choice([1e-5, 1e-6])), "groups": groups}, "canon": {"taps": int(rng.integers(1, 6))},
+            "embedding": {"scale": float(rng.choice([1.0, width ** 0.5]))}, "layers": layers}
