@@ -940,3 +940,241 @@ class ZedudraConfig(ModelConfig):
         if self.max_position_embeddings != (1 << 24):
             d["max_position_embeddings"] = self.max_position_embeddings
         return d
+
+
+# ---------------------------------------------------------------------------------------
+# Furanex
+# ---------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class FuranexRotation:
+    """Rotation by position over the first ``dims`` channels; ``stretch`` = (factor, original, fast, slow) slows the
+    low frequencies down for contexts longer than ``original`` (None: plain frequencies)."""
+    dims: int
+    base: float
+    stretch: Optional[Tuple[float, float, float, float]] = None
+
+    def to_dict(self) -> Dict[str, Any]:
+        d: Dict[str, Any] = {"dims": self.dims, "base": self.base}
+        if self.stretch is not None:
+            d["scaling"] = dict(zip(("factor", "original", "fast", "slow"), self.stretch))
+        return d
+
+
+@dataclass(frozen=True)
+class FuranexMixer:
+    """``kind`` "attention": ``heads`` query heads on ``kv_heads`` key/value heads, keys of ``dim`` and values of ``vdim``
+    channels, ``v_mix``: the values are shared along the layers. ``kind`` "latent_attention": ``heads`` heads with ``dim``
+    unrotated and ``rot_dim`` rotated query/key channels, values of ``vdim``, latents of ``q_rank`` and ``kv_rank``."""
+    kind: str
+    heads: int
+    dim: int
+    vdim: int
+    scale: float
+    rot: Optional[FuranexRotation] = None
+    kv_heads: int = 0
+    v_mix: bool = False
+    rot_dim: int = 0
+    q_rank: int = 0
+    kv_rank: int = 0
+
+    def to_dict(self) -> Dict[str, Any]:
+        d: Dict[str, Any] = {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale}
+        if self.rot is not None:
+            d["rot"] = self.rot.to_dict()
+        if self.kind == "attention":
+            d.update(kv_heads=self.kv_heads, v_mix=self.v_mix)
+        else:
+            d.update(rot_dim=self.rot_dim, q_rank=self.q_rank, kv_rank=self.kv_rank)
+        return d
+
+
+@dataclass(frozen=True)
+class FuranexFeedForward:
+    """A mixture of ``experts`` gated pairs of width ``ff`` of which a token uses ``top``, named by a stored table from
+    its token id; ``shared_ff`` > 0: a shared expert of that width beside them."""
+    ff: int
+    experts: int
+    top: int
+    shared_ff: int = 0
+
+    def to_dict(self) -> Dict[str, Any]:
+        d: Dict[str, Any] = {"kind": "moe", "expert": {"ff": self.ff}, "router": {"experts": self.experts, "top": self.top}}
+        if self.shared_ff:
+            d["shared"] = {"ff": self.shared_ff}
+        return d
+
+
+@dataclass(frozen=True)
+class FuranexLayer:
+    mixer: FuranexMixer
+    mlp: Optional[FuranexFeedForward] = None
+
+
+@dataclass(frozen=True)
+class FuranexConfig(ModelConfig):
+    """Furanex: a pre-norm decoder on several residual streams (``streams``) whose ``layers`` are listed one by one: grouped
+    softmax attention (rotation first, then a unit norm of q and k; values blended with the first such layer's) or
+    attention over a cached latent with a gate per head; feed-forwards whose experts a table names by token id, beside a
+    shared expert. The embedding is multiplied by ``embedding.scale``; the output head is the embedding's table.
+    Keys: ``vocab``, ``width``, ``streams``, ``layers``, ``norm.eps``, ``embedding.scale``."""
+
+    architecture: ClassVar[str] = "Furanex"
+
+    vocab_size: int = 0
+    hidden_size: int = 0
+    streams: int = 0                       # 0: one plain residual
+    layers: Tuple[FuranexLayer, ...] = ()
+    norm_eps: float = 1e-6
+    embedding_scale: float = 1.0
+    max_position_embeddings: int = 1 << 24
+    dtype: str = "bfloat16"
+    eos_token_ids: Tuple[int, ...] = ()
+
+    @staticmethod
+    def _rotation(m: Dict[str, Any], mw: str) -> Optional[FuranexRotation]:
+        rot = _section(m, "rot", mw, optional=True)
+        if rot is None:
+            return None
+        rw = mw + ".rot"
+        sc = _section(rot, "scaling", rw, optional=True)
+        stretch = None
+        if sc is not None:
+            stretch = tuple(_require(sc, k, float, rw + ".scaling") for k in ("factor", "original", "fast", "slow"))
+        return FuranexRotation(dims=_require(rot, "dims", int, rw), base=_require(rot, "base", float, rw), stretch=stretch)
+
+    @classmethod
+    def from_dict(cls, d: Dict[str, Any], where: str = "config.json") -> "FuranexConfig":
+        raw_layers = d.get("layers")
+        if not isinstance(raw_layers, (list, tuple)) or not raw_layers:
+            raise ConfigError(f"{where}: 'layers' must be a non-empty list")
+        layers = []
+        for i, entry in enumerate(raw_layers):
+            lw = f"{where}: layers[{i}]"
+            if not isinstance(entry, dict):
+                raise ConfigError(f"{lw} must be an object")
+            kind = entry.get("type")
+            m = _section(entry, "mixer", lw)
+            mw = lw + ".mixer"
+            heads, dim = _require(m, "heads", int, mw), _require(m, "dim", int, mw)
+            vdim, scale = m.get("vdim"), m.get("scale")
+            rot = cls._rotation(m, mw)
+            common = dict(kind=kind, heads=heads, dim=dim, vdim=dim if vdim is None else _typed(vdim, "vdim", int, mw), rot=rot)
+            if kind == "attention":
+                kv_heads, v_mix = m.get("kv_heads"), m.get("v_mix")
+                mixer = FuranexMixer(scale=dim ** -0.5 if scale is None else _typed(scale, "scale", float, mw),
+                                     kv_heads=heads if kv_heads is None else _typed(kv_heads, "kv_heads", int, mw),
+                                     v_mix=False if v_mix is None else _typed(v_mix, "v_mix", bool, mw), **common)
+            elif kind == "latent_attention":
+                rot_dim = m.get("rot_dim")
+                rot_dim = (rot.dims if rot is not None else 0) if rot_dim is None else _typed(rot_dim, "rot_dim", int, mw)
+                mixer = FuranexMixer(scale=(dim + rot_dim) ** -0.5 if scale is None else _typed(scale, "scale", float, mw),
+                                     rot_dim=rot_dim, q_rank=_require(m, "q_rank", int, mw),
+                                     kv_rank=_require(m, "kv_rank", int, mw), **common)
+            else:
+                raise ConfigError(f"{lw}: layer type {kind!r} is not supported (attention, latent_attention)")
+            mlp = _section(entry, "mlp", lw, optional=True)
+            ff = None
+            if mlp is not None:
+                pw = lw + ".mlp"
+                if mlp.get("kind", "moe") != "moe":
+                    raise ConfigError(f"{pw}: kind {mlp.get('kind')!r} is not supported (moe)")
+                expert = _section(mlp, "expert", pw)
+                router = _section(mlp, "router", pw)
+                shared = _section(mlp, "shared", pw, optional=True)
+                ff = FuranexFeedForward(ff=_require(expert, "ff", int, pw + ".expert"),
+                                        experts=_require(router, "experts", int, pw + ".router"),
+                                        top=_require(router, "top", int, pw + ".router"),
+                                        shared_ff=0 if shared is None else _require(shared, "ff", int, pw + ".shared"))
+            layers.append(FuranexLayer(mixer=mixer, mlp=ff))
+        norm = _section(d, "norm", where)
+        emb = _section(d, "embedding", where, optional=True)
+        emb_scale = None if emb is None else emb.get("scale")
+        streams = d.get("streams")
+        dtype = d.get("dtype", d.get("torch_dtype", "bfloat16")) or "bfloat16"
+        if str(dtype) not in _DTYPE_NAMES:
+            raise ConfigError(f"{where}: unknown dtype {dtype!r}")
+        eos = d.get("eos_token_id")
+        eos_ids: Tuple[int, ...] = ()
+        if isinstance(eos, int) and not isinstance(eos, bool):
+            eos_ids = (eos,)
+        elif isinstance(eos, (list, tuple)) and all(isinstance(e, int) for e in eos):
+            eos_ids = tuple(eos)
+        elif eos is not None:
+            raise ConfigError(f"{where}: eos_token_id must be an integer or a list of integers, got {eos!r}")
+        max_pos = d.get("max_position_embeddings")
+        cfg = cls(
+            vocab_size=_require(d, "vocab", int, where),
+            hidden_size=_require(d, "width", int, where),
+            streams=0 if streams is None else _typed(streams, "streams", int, where),
+            layers=tuple(layers),
+            norm_eps=_require(norm, "eps", float, where + ".norm"),
+            embedding_scale=1.0 if emb_scale is None else _typed(emb_scale, "scale", float, where + ".embedding"),
+            max_position_embeddings=(1 << 24) if max_pos is None else _typed(max_pos, "max_position_embeddings", int, where),
+            dtype=_DTYPE_NAMES[str(dtype)],
+            eos_token_ids=eos_ids,
+        )
+        cfg.validate(where)
+        return cfg
+
+    def first_mixing_layer(self) -> Optional[int]:
+        """The first attention layer whose values are shared along the layers: the others blend its values into theirs."""
+        for i, l in enumerate(self.layers):
+            if l.mixer.kind == "attention" and l.mixer.v_mix:
+                return i
+        return None
+
+    def validate(self, where: str = "config") -> None:
+        if self.vocab_size <= 0 or self.hidden_size <= 0:
+            raise ConfigError(f"{where}: vocab and width must be positive")
+        if self.norm_eps <= 0:
+            raise ConfigError(f"{where}: norm.eps must be positive, got {self.norm_eps}")
+        if self.streams < 0 or self.streams > 8:
+            raise ConfigError(f"{where}: streams must lie in 1..8, got {self.streams}")
+        first = self.first_mixing_layer()
+        for i, l in enumerate(self.layers):
+            lw = f"{where}: layers[{i}]"
+            m = l.mixer
+            if m.heads <= 0 or m.dim <= 0 or m.vdim <= 0 or not m.scale > 0:
+                raise ConfigError(f"{lw}: heads, dim, vdim and scale must be positive")
+            if m.rot is not None:
+                r = m.rot
+                if r.dims <= 0 or r.dims % 2 or not r.base > 1:
+                    raise ConfigError(f"{lw}: rot.dims {r.dims} must be positive and even, rot.base above 1")
+                if r.stretch is not None and not all(v > 0 for v in r.stretch):
+                    raise ConfigError(f"{lw}: rot.scaling needs positive factor, original, fast and slow")
+            if m.kind == "attention":
+                if m.kv_heads <= 0 or m.heads % m.kv_heads:
+                    raise ConfigError(f"{lw}: {m.heads} heads are not a multiple of {m.kv_heads} kv_heads")
+                if m.rot is not None and m.rot.dims > m.dim:
+                    raise ConfigError(f"{lw}: rot.dims {m.rot.dims} exceeds dim {m.dim}")
+                if m.v_mix and (self.layers[first].mixer.kv_heads, self.layers[first].mixer.vdim) != (m.kv_heads, m.vdim):
+                    raise ConfigError(f"{lw}: layers that share their values need the kv_heads and vdim of layer {first}")
+            else:
+                if m.q_rank <= 0 or m.kv_rank <= 0 or m.rot_dim < 0 or m.rot_dim % 2:
+                    raise ConfigError(f"{lw}: q_rank and kv_rank must be positive, rot_dim even and >= 0")
+                if (m.rot.dims if m.rot is not None else 0) != m.rot_dim:
+                    raise ConfigError(f"{lw}: the rotated part has rot_dim {m.rot_dim} channels, so rot.dims must equal it")
+            f = l.mlp
+            if f is not None:
+                if f.ff <= 0 or f.experts < 1 or not (1 <= f.top <= f.experts) or f.shared_ff < 0:
+                    raise ConfigError(f"{lw}: a mixture needs a positive expert width, experts >= 1 and 1 <= top <= experts")
+
+    def to_dict(self) -> Dict[str, Any]:
+        layers = [{"type": l.mixer.kind, "mixer": l.mixer.to_dict(), "mlp": None if l.mlp is None else l.mlp.to_dict()}
+                  for l in self.layers]
+        d: Dict[str, Any] = {
+            "architecture": self.architecture,
+            "layers": layers,
+            "norm": {"eps": self.norm_eps},
+            "embedding": {"scale": self.embedding_scale},
+            "vocab": self.vocab_size,
+            "width": self.hidden_size,
+            "torch_dtype": self.dtype,
+        }
+        if self.streams:
+            d["streams"] = self.streams
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids) if len(self.eos_token_ids) > 1 else self.eos_token_ids[0]
+        if self.max_position_embeddings != (1 << 24):
+            d["max_position_embeddings"] = self.max_position_embeddings
+        return d

@@ -29,11 +29,13 @@ def named_shapes() -> Dict[str, Dict[str, Any]]:
     shapes["bolapel-tiny"] = bolapel_tiny_shape()
     shapes["dutilix-tiny"] = dutilix_tiny_shape()
     shapes["zedudra-tiny"] = zedudra_tiny_shape()
+    shapes["furanex-tiny"] = furanex_tiny_shape()
     for name in QWEN3_SHAPES:
         if name != "tiny":
             shapes[f"bolapel-{name}"] = bolapel_shape(name)
             shapes[f"dutilix-{name}"] = dutilix_shape(name)
             shapes[f"zedudra-{name}"] = zedudra_shape(name)
+            shapes[f"furanex-{name}"] = furanex_shape(name)
     return shapes
 
 
@@ -174,3 +176,43 @@ def zedudra_tiny_shape() -> Dict[str, Any]:
                        {"type": "attention", "mixer": dict(mixer), "mlp": moe},
                        {"type": "attention", "mixer": dict(mixer), "mlp": moe, "weights_of": 1},
                        {"type": "attention", "mixer": dict(mixer, kv_heads=4), "mlp": None}]}
+
+
+def furanex_shape(name: str, layers: int = None, streams: int = 4, experts: int = 32, top: int = 4, shared: bool = True,
+                  latent_every: int = 2) -> Dict[str, Any]:
+    """A Furanex configuration with the width, vocabulary, head counts, head size and number of layers of the named Qwen3
+    shape: every ``latent_every``-th layer (from the second) is attention over a latent of 256 with 64 rotated channels
+    and a query latent of a quarter of the width, the others are grouped attention whose values are shared along the
+    layers; every feed-forward is a mixture of ``experts`` experts of which ``top`` are used, each 1/top of the shape's
+    dense width, beside a shared expert of the same size. For random-weights models at sizes that resemble a real
+    model's layers."""
+    q = QWEN3_SHAPES[name]
+    n = layers or q["num_hidden_layers"]
+    hid, hd = q["hidden_size"], q["head_dim"]
+    stretch = {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+    attention = {"heads": q["num_attention_heads"], "kv_heads": q["num_key_value_heads"], "dim": hd, "vdim": hd,
+                 "scale": 0.125, "v_mix": True, "rot": {"dims": hd, "base": q["rope_theta"], "scaling": dict(stretch)}}
+    latent = {"heads": q["num_attention_heads"], "dim": hd, "rot_dim": 64, "vdim": hd, "q_rank": max(64, hid // 4),
+              "kv_rank": 256, "scale": (hd + 64) ** -0.5, "rot": {"dims": 64, "base": 10000.0, "scaling": dict(stretch)}}
+    mlp = {"kind": "moe", "expert": {"ff": q["intermediate_size"] // top}, "router": {"experts": experts, "top": top}}
+    if shared:
+        mlp["shared"] = {"ff": q["intermediate_size"] // top}
+    out = [{"type": "latent_attention" if i % latent_every == latent_every - 1 else "attention",
+            "mixer": dict(latent if i % latent_every == latent_every - 1 else attention), "mlp": dict(mlp)} for i in range(n)]
+    return {"architecture": "Furanex", "vocab": q["vocab_size"], "width": hid, "streams": streams, "layers": out,
+            "norm": {"eps": q["rms_norm_eps"]}, "embedding": {"scale": float(hid) ** 0.5}}
+
+
+def furanex_tiny_shape() -> Dict[str, Any]:
+    """A Furanex model of a few thousand weights: two value-sharing attention layers around a latent-attention layer,
+    one of them without a feed-forward."""
+    stretch = {"factor": 3.0, "original": 64, "fast": 16.0, "slow": 2.0}
+    attention = {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 8, "scale": 0.2, "v_mix": True,
+                 "rot": {"dims": 12, "base": 5000.0, "scaling": dict(stretch)}}
+    latent = {"heads": 3, "dim": 12, "rot_dim": 4, "vdim": 8, "q_rank": 24, "kv_rank": 16, "scale": 0.25,
+              "rot": {"dims": 4, "base": 10000.0, "scaling": dict(stretch)}}
+    moe = {"kind": "moe", "expert": {"ff": 24}, "router": {"experts": 5, "top": 2}, "shared": {"ff": 40}}
+    return {"architecture": "Furanex", "vocab": 256, "width": 48, "streams": 3, "norm": {"eps": 1e-5}, "embedding": {"scale": 6.0},
+            "layers": [{"type": "attention", "mixer": dict(attention), "mlp": dict(moe)},
+                       {"type": "latent_attention", "mixer": dict(latent), "mlp": None},
+                       {"type": "attention", "mixer": dict(attention), "mlp": dict(moe)}]}

@@ -93,7 +93,7 @@ extern "C" int mv_latent_prepare(const void* packed, long ld, int n, int QR, int
 // y rows [n][H][ldy_head]:  y[t][h][j] = sum_i x[t][h][i] w[h][i][j], the sum in the order of i.
 //   tail > 0   x[t][h][IN .. IN+tail) is copied behind the OUT outputs, rotated by the row's position
 //              (pairs i, i + tail/2; table[p] = [cos | sin])
-//   gate       y is multiplied by sigmoid(gate[t][h * OUT + j])
+//   gate       y is multiplied by sigmoid(gate[t][h * OUT + j]), or by sigmoid(gate[t][h]) with `gate_per_head`
 // ---------------------------------------------------------------------------------------
 #define HL_TOKENS 8
 #define HL_MAX_IN 1024
@@ -107,7 +107,7 @@ template <typename TIN, typename TOUT, typename TG, int HL_COLS, int HL_SLICES>
 __global__ void __launch_bounds__(256)
 head_linear_kernel(const TIN* __restrict__ x, long ldx, int ldx_head, WeightPtr w, int IN, int OUT, TOUT* __restrict__ y, long ldy,
                    int ldy_head, int tail, const float* __restrict__ table, const int* __restrict__ positions,
-                   const TG* __restrict__ gate, long ldg, const int* __restrict__ token_seq, int n) {
+                   const TG* __restrict__ gate, long ldg, int gate_per_head, const int* __restrict__ token_seq, int n) {
     __shared__ float xs[HL_TOKENS][HL_MAX_IN];
     __shared__ float part[HL_SLICES][HL_TOKENS][HL_COLS];
     const int t0 = blockIdx.x * HL_TOKENS, head = blockIdx.y, tid = threadIdx.x;
@@ -151,7 +151,7 @@ head_linear_kernel(const TIN* __restrict__ x, long ldx, int ldx_head, WeightPtr 
 #pragma unroll
         for (int sl = 0; sl < HL_SLICES; ++sl) v += part[sl][tt][c];
         if (token_seq[t0 + tt] < 0) v = 0.f;
-        else if (gate) v *= 1.f / (1.f + expf(-to_f(gate[(size_t)(t0 + tt) * ldg + (size_t)head * OUT + jj])));
+        else if (gate) v *= 1.f / (1.f + expf(-to_f(gate[(size_t)(t0 + tt) * ldg + (gate_per_head ? (size_t)head : (size_t)head * OUT + jj)])));
         y[(size_t)(t0 + tt) * ldy + (size_t)head * ldy_head + jj] = from_f<TOUT>(v);
     }
     if (blockIdx.z != 0) return;
@@ -177,13 +177,13 @@ head_linear_kernel(const TIN* __restrict__ x, long ldx, int ldx_head, WeightPtr 
 // type (with an optional gate of the activation type)
 extern "C" int mv_head_linear(const void* x, long ldx, int ldx_head, const void* w, int weight_dtype, int n, int H, int IN,
                               int OUT, void* y, long ldy, int ldy_head, int tail, const float* table, const int* positions,
-                              const void* gate, long ldg, const int* token_seq, int mode, int dtype, hipStream_t stream) {
+                              const void* gate, long ldg, int gate_per_head, const int* token_seq, int mode, int dtype, hipStream_t stream) {
     MV_REQUIRE(n >= 0 && H > 0 && IN > 0 && OUT > 0 && tail >= 0 && tail % 2 == 0, "head_linear: bad sizes n=%d H=%d IN=%d OUT=%d", n, H, IN, OUT);
     MV_REQUIRE(IN <= HL_MAX_IN, "head_linear: %d inputs a head, at most %d are served", IN, HL_MAX_IN);
     MV_REQUIRE(ldx_head >= IN + tail && ldy_head >= OUT + tail && ldx >= (long)(H - 1) * ldx_head + IN + tail
                && ldy >= (long)(H - 1) * ldy_head + OUT + tail, "head_linear: row pitches too small");
     MV_REQUIRE(mv_valid_dtype(weight_dtype) && x && w && y && token_seq && (tail == 0 || (table && positions)) && H <= 65535
-               && (!gate || ldg >= (long)H * OUT), "head_linear: missing operand");
+               && (!gate || ldg >= (gate_per_head ? (long)H : (long)H * OUT)), "head_linear: missing operand");
     MV_REQUIRE((mode == 0 && !gate) || (mode == 1 && tail == 0), "head_linear: mode %d does not take these options", mode);
     if (n == 0) return 0;
     WeightPtr wp{w, weight_dtype};
@@ -195,12 +195,12 @@ extern "C" int mv_head_linear(const void* x, long ldx, int ldx_head, const void*
         MV_DISPATCH_T(dtype, "head_linear",                                                                                 \
                       hipLaunchKernelGGL((head_linear_kernel<T, float, T, C, S>), grid, dim3(256), 0, stream, (const T*)x, ldx, \
                                          ldx_head, wp, IN, OUT, (float*)y, ldy, ldy_head, tail, table, positions,           \
-                                         (const T*)nullptr, 0L, token_seq, n));                                             \
+                                         (const T*)nullptr, 0L, 0, token_seq, n));                                             \
     } else {                                                                                                                \
         MV_DISPATCH_T(dtype, "head_linear",                                                                                 \
                       hipLaunchKernelGGL((head_linear_kernel<float, T, T, C, S>), grid, dim3(256), 0, stream, (const float*)x,  \
                                          ldx, ldx_head, wp, IN, OUT, (T*)y, ldy, ldy_head, 0, table, positions,             \
-                                         (const T*)gate, ldg, token_seq, n));                                               \
+                                         (const T*)gate, ldg, gate_per_head, token_seq, n));                                               \
     }
     if (few) {
         HL_LAUNCH(16, 16)
@@ -766,7 +766,7 @@ template <int MODE>
 __global__ void __launch_bounds__(256)
 head_linear_mfma_kernel(const void* __restrict__ xv, long ldx, int ldx_head, const bf16* __restrict__ w, int IN, int OUT,
                         void* __restrict__ yv, long ldy, int ldy_head, int tail, const float* __restrict__ table,
-                        const int* __restrict__ positions, const bf16* __restrict__ gate, long ldg,
+                        const int* __restrict__ positions, const bf16* __restrict__ gate, long ldg, int gate_per_head,
                         const int* __restrict__ token_seq, int n) {
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int t0 = blockIdx.x * 64 + 16 * wave, head = blockIdx.y, n0 = blockIdx.z * 128;
@@ -816,7 +816,7 @@ head_linear_mfma_kernel(const void* __restrict__ xv, long ldx, int ldx_head, con
             if (MODE == 0) {
                 ((float*)yv)[(size_t)t * ldy + (size_t)head * ldy_head + col] = v;
             } else {
-                if (gate && !pad) v *= 1.f / (1.f + expf(-to_f(gate[(size_t)t * ldg + (size_t)head * OUT + col])));
+                if (gate && !pad) v *= 1.f / (1.f + expf(-to_f(gate[(size_t)t * ldg + (gate_per_head ? (size_t)head : (size_t)head * OUT + col)])));
                 ((bf16*)yv)[(size_t)t * ldy + (size_t)head * ldy_head + col] = from_f<bf16>(v);
             }
         }
@@ -844,7 +844,7 @@ head_linear_mfma_kernel(const void* __restrict__ xv, long ldx, int ldx_head, con
 // returns 2 (nothing done) for sizes it does not serve
 extern "C" int mv_head_linear_mfma(const void* x, long ldx, int ldx_head, const void* w, int n, int H, int IN, int OUT, void* y,
                                    long ldy, int ldy_head, int tail, const float* table, const int* positions, const void* gate,
-                                   long ldg, const int* token_seq, int mode, hipStream_t stream) {
+                                   long ldg, int gate_per_head, const int* token_seq, int mode, hipStream_t stream) {
     MV_REQUIRE(n >= 0 && H > 0 && IN > 0 && OUT > 0 && tail >= 0 && tail % 2 == 0, "head_linear_mfma: bad sizes");
     if (IN % 32 != 0 || ((uintptr_t)w % 16) != 0 || (mode == 1 && (ldx % 4 || ldx_head % 4))) return 2;
     MV_REQUIRE(ldx_head >= IN + tail && ldy_head >= OUT + (mode == 0 ? tail : 0) && x && w && y && token_seq && H <= 65535
@@ -853,10 +853,10 @@ extern "C" int mv_head_linear_mfma(const void* x, long ldx, int ldx_head, const 
     dim3 grid((n + 63) / 64, H, (OUT + 127) / 128);
     if (mode == 0)
         hipLaunchKernelGGL(head_linear_mfma_kernel<0>, grid, dim3(256), 0, stream, x, ldx, ldx_head, (const bf16*)w, IN, OUT, y, ldy,
-                           ldy_head, tail, table, positions, (const bf16*)nullptr, 0L, token_seq, n);
+                           ldy_head, tail, table, positions, (const bf16*)nullptr, 0L, 0, token_seq, n);
     else
         hipLaunchKernelGGL(head_linear_mfma_kernel<1>, grid, dim3(256), 0, stream, x, ldx, ldx_head, (const bf16*)w, IN, OUT, y, ldy,
-                           ldy_head, 0, table, positions, (const bf16*)gate, ldg, token_seq, n);
+                           ldy_head, 0, table, positions, (const bf16*)gate, ldg, gate_per_head, token_seq, n);
     return mv_check_launch("head_linear_mfma");
 }
 #endif

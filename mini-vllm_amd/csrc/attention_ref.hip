@@ -10,7 +10,7 @@
 // `first`, never on how the step was batched. With `gate`, head h's output row is multiplied by
 // sigmoid(gate[token][h]).
 //
-// Layouts:  K[page][kv_head][slot][d]   V[page][kv_head][d][slot]
+// Layouts:  K[page][kv_head][slot][d]   V[page][kv_head][dv][slot]   (a value row may have another size, Dv, than a key's)
 // This kernel takes every head size up to 512 and every page size; it is the float32
 // path's attention and the fall-back of the bfloat16 path.
 #include "dispatch.h"
@@ -23,7 +23,7 @@ __global__ void __launch_bounds__(AR_THREADS)
 attention_ref_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out, long out_stride,
                      const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                      const int* __restrict__ block_table, int bt_width, int page_size,
-                     const int* __restrict__ positions, const int* __restrict__ token_seq, int H, int Hkv, int D,
+                     const int* __restrict__ positions, const int* __restrict__ token_seq, int H, int Hkv, int D, int Dv,
                      float scale, int window, int first, const T* __restrict__ gate, long gate_stride) {
     __shared__ float qs[AR_MAX_D];
     __shared__ float ps[AR_THREADS];
@@ -34,9 +34,9 @@ attention_ref_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out
     const int head = blockIdx.y;
     const int tid = threadIdx.x;
     const int seq = token_seq[tok];
-    T* o = out + (size_t)tok * out_stride + (size_t)head * D;
+    T* o = out + (size_t)tok * out_stride + (size_t)head * Dv;
     if (seq < 0) {
-        for (int d = tid; d < D; d += AR_THREADS) o[d] = from_f<T>(0.f);
+        for (int d = tid; d < Dv; d += AR_THREADS) o[d] = from_f<T>(0.f);
         return;
     }
     const int pos = positions[tok];
@@ -71,7 +71,7 @@ attention_ref_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out
             float dot = 0.f;
             for (int d = 0; d < D; ++d) dot = fmaf(qs[d], to_f(krow[d]), dot);
             s = dot * scale;
-            vo = (long)(((size_t)page * Hkv + kvh) * D) * page_size + slot;
+            vo = (long)(((size_t)page * Hkv + kvh) * Dv) * page_size + slot;
         }
         const float tmax = block_max(s, scratch);
         const float m_new = fmaxf(m, tmax);
@@ -86,7 +86,7 @@ attention_ref_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out
 #pragma unroll
         for (int i = 0; i < AR_MAX_D / AR_THREADS; ++i) {
             const int d = tid + i * AR_THREADS;
-            if (d < D) {
+            if (d < Dv) {
                 float a = acc[i] * corr;
                 for (int jj = 0; jj < cnt; ++jj)
                     a = fmaf(ps[jj], to_f(v_pages[voff[jj] + (long)d * page_size]), a);
@@ -100,28 +100,28 @@ attention_ref_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out
 #pragma unroll
     for (int i = 0; i < AR_MAX_D / AR_THREADS; ++i) {
         const int d = tid + i * AR_THREADS;
-        if (d < D) o[d] = from_f<T>(acc[i] * inv);
+        if (d < Dv) o[d] = from_f<T>(acc[i] * inv);
     }
 }
 
 extern "C" int mv_attention_ref(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
                                 const void* v_pages, const int* block_table, int bt_width, int page_size,
-                                const int* positions, const int* token_seq, int n, int H, int Hkv, int D,
+                                const int* positions, const int* token_seq, int n, int H, int Hkv, int D, int Dv,
                                 float scale, int window, int first, const void* gate, long gate_stride, int dtype,
                                 hipStream_t stream) {
     MV_REQUIRE(n >= 0 && H > 0 && Hkv > 0 && D > 0, "attention: bad sizes n=%d H=%d Hkv=%d D=%d", n, H, Hkv, D);
     MV_REQUIRE(H % Hkv == 0, "attention: %d query heads are not a multiple of %d key/value heads", H, Hkv);
-    MV_REQUIRE(D <= AR_MAX_D, "attention: head_dim %d exceeds the supported maximum %d", D, AR_MAX_D);
+    MV_REQUIRE(D <= AR_MAX_D && Dv > 0 && Dv <= AR_MAX_D, "attention: head sizes %d / %d exceed the supported maximum %d", D, Dv, AR_MAX_D);
     MV_REQUIRE(page_size > 0 && bt_width > 0, "attention: bad page size %d or block table width %d", page_size,
                bt_width);
-    MV_REQUIRE(q_stride >= (long)H * D && out_stride >= (long)H * D, "attention: row strides too small");
+    MV_REQUIRE(q_stride >= (long)H * D && out_stride >= (long)H * Dv, "attention: row strides too small");
     MV_REQUIRE(H <= 65535, "attention: too many heads %d", H);
     MV_REQUIRE(first >= 0 && (gate == nullptr || gate_stride >= H), "attention: bad count of kept first positions or gate rows too short");
     if (n == 0) return 0;
     MV_DISPATCH_T(dtype, "attention",
                   hipLaunchKernelGGL(attention_ref_kernel<T>, dim3(n, H), dim3(AR_THREADS), 0, stream, (const T*)q,
                                      q_stride, (T*)out, out_stride, (const T*)k_pages, (const T*)v_pages,
-                                     block_table, bt_width, page_size, positions, token_seq, H, Hkv, D, scale,
+                                     block_table, bt_width, page_size, positions, token_seq, H, Hkv, D, Dv, scale,
                                      window, first, (const T*)gate, gate_stride));
     return mv_check_launch("attention");
 }

@@ -27,7 +27,7 @@ ARCH = "gfx950"
 
 # translation units of each variant
 COMMON_SOURCES = ["runtime.hip", "elementwise.hip", "gemm_ref.hip", "attention_ref.hip", "sampling.hip", "recurrent.hip",
-                  "attention_sigmoid.hip", "attention_latent.hip", "moe.hip", "group_norm.hip"]
+                  "attention_sigmoid.hip", "attention_latent.hip", "moe.hip", "group_norm.hip", "hyper.hip", "qkv_rotate.hip"]
 VARIANT_SOURCES: Dict[str, List[str]] = {
     "f32": COMMON_SOURCES,
     "bf16": COMMON_SOURCES + ["gemm_skinny.hip", "gemm_mid.hip", "gemm_tile.hip", "gemm_lt.hip", "attention_fast.hip",

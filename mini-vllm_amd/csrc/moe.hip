@@ -145,19 +145,22 @@ extern "C" int mv_moe_route(const float* logits, long ld, int n, int E, const vo
     return mv_check_launch("moe_route");
 }
 
-// gate_up rows: [gate of expert 0 (F) | ... | gate of expert E-1 | up of expert 0 | ... ]; act rows [E][F]
+// gate_up rows: [gate of expert 0 (F) | ... | gate of expert E-1 | up of expert 0 | ... | up of expert E-1 | gate of the
+// shared expert (FS) | its up (FS)]; act rows [E][F] and behind them the shared expert's FS, whose weight is one
 template <typename T>
 __global__ void __launch_bounds__(256)
-moe_swiglu_scale_kernel(const T* __restrict__ gate_up, long ld, const float* __restrict__ dense, int ld_dense, int E, int F,
+moe_swiglu_scale_kernel(const T* __restrict__ gate_up, long ld, const float* __restrict__ dense, int ld_dense, int E, int F, int FS,
                         T* __restrict__ act, long total, float limit, float slope) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const long EF = (long)E * F;
-    const long t = i / EF, c = i % EF;
-    const float w = dense[t * ld_dense + c / F];
+    const long t = i / (EF + FS), c = i % (EF + FS);
+    const bool shared = c >= EF;
+    const float w = shared ? 1.f : dense[t * ld_dense + c / F];
     float v = 0.f;
     if (w != 0.f) {
-        const float g = to_f(gate_up[t * ld + c]), u = to_f(gate_up[t * ld + EF + c]);
+        const long gi = shared ? 2 * EF + (c - EF) : c, ui = shared ? 2 * EF + FS + (c - EF) : EF + c;
+        const float g = to_f(gate_up[t * ld + gi]), u = to_f(gate_up[t * ld + ui]);
         if (limit > 0.f) {
             const float gc = fminf(g, limit), uc = fminf(fmaxf(u, -limit), limit);
             v = w * (gc / (1.f + expf(-slope * gc))) * (uc + 1.f);
@@ -165,19 +168,56 @@ moe_swiglu_scale_kernel(const T* __restrict__ gate_up, long ld, const float* __r
             v = w * (g / (1.f + expf(-g))) * u;
         }
     }
-    act[t * EF + c] = from_f<T>(v);
+    act[t * (EF + FS) + c] = from_f<T>(v);
 }
 
-extern "C" int mv_moe_swiglu_scale(const void* gate_up, long ld, const float* dense, int ld_dense, int n, int E, int F, void* act,
-                                   float limit, float slope, int dtype, hipStream_t stream) {
-    MV_REQUIRE(n >= 0 && E > 0 && F > 0 && ld >= 2L * E * F && ld_dense >= E, "moe_swiglu_scale: bad sizes n=%d E=%d F=%d", n, E, F);
+extern "C" int mv_moe_swiglu_scale(const void* gate_up, long ld, const float* dense, int ld_dense, int n, int E, int F, int FS,
+                                   void* act, float limit, float slope, int dtype, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && E > 0 && F > 0 && FS >= 0 && ld >= 2L * E * F + 2L * FS && ld_dense >= E,
+               "moe_swiglu_scale: bad sizes n=%d E=%d F=%d shared=%d", n, E, F, FS);
     MV_REQUIRE(gate_up && dense && act, "moe_swiglu_scale: missing operand");
-    const long total = (long)n * E * F;
+    const long total = (long)n * ((long)E * F + FS);
     if (total == 0) return 0;
     MV_DISPATCH_T(dtype, "moe_swiglu_scale",
                   hipLaunchKernelGGL(moe_swiglu_scale_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
-                                     (const T*)gate_up, ld, dense, ld_dense, E, F, (T*)act, total, limit, slope));
+                                     (const T*)gate_up, ld, dense, ld_dense, E, F, FS, (T*)act, total, limit, slope));
     return mv_check_launch("moe_swiglu_scale");
+}
+
+// Experts named by a table instead of a router: row t uses table[ids[t]][0 .. top), each with the weight 1 / top.
+// Leaves what moe_route leaves: dense [n][ld_dense] (the first E columns; zeros for the others), ids and weights
+// [n][top] in the table's order. A token id outside the table, and an entry outside the experts, choose nothing.
+__global__ void __launch_bounds__(64)
+moe_table_route_kernel(const int* __restrict__ tokens, const int* __restrict__ table, int rows, int E, int top,
+                       float* __restrict__ dense, int ld_dense, int* __restrict__ ids, float* __restrict__ weights) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const int tok = tokens[t];
+    const bool known = tok >= 0 && tok < rows;
+    const float w = 1.f / (float)top;
+    for (int e = lane; e < E; e += 64) {
+        float v = 0.f;
+        if (known)
+            for (int k = 0; k < top; ++k)
+                if (table[(size_t)tok * top + k] == e) v += w;
+        dense[(size_t)t * ld_dense + e] = v;
+    }
+    for (int k = lane; k < top; k += 64) {
+        const int e = known ? table[(size_t)tok * top + k] : -1;
+        const bool ok = e >= 0 && e < E;
+        ids[(size_t)t * top + k] = ok ? e : -1;
+        weights[(size_t)t * top + k] = ok ? w : 0.f;
+    }
+}
+
+extern "C" int mv_moe_table_route(const int* tokens, const int* table, int rows, int n, int E, int top, float* dense,
+                                  int ld_dense, int* ids, float* weights, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && rows > 0 && E > 0 && top > 0 && top <= E && ld_dense >= E, "moe_table_route: bad sizes n=%d rows=%d E=%d top=%d",
+               n, rows, E, top);
+    MV_REQUIRE(tokens && table && dense && ids && weights, "moe_table_route: missing operand");
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(moe_table_route_kernel, dim3(n), dim3(64), 0, stream, tokens, table, rows, E, top, dense, ld_dense, ids,
+                       weights);
+    return mv_check_launch("moe_table_route");
 }
 
 template <typename T>
@@ -205,6 +245,26 @@ extern "C" int mv_moe_identity_add(void* y, long ldy, const void* h, long ldh, c
                   hipLaunchKernelGGL(moe_identity_add_kernel<T>, dim3(n), dim3(256), 0, stream, (T*)y, ldy, (const T*)h, ldh, dense,
                                      ld_dense, first, count, width, set));
     return mv_check_launch("moe_identity_add");
+}
+
+// rows of the activation type: y <- y + x, added in float
+template <typename T>
+__global__ void __launch_bounds__(256)
+add_rows_kernel(T* __restrict__ y, long ldy, const T* __restrict__ x, long ldx, int cols, long total) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    T* p = y + (i / cols) * ldy + (i % cols);
+    *p = from_f<T>(to_f(*p) + to_f(x[(i / cols) * ldx + (i % cols)]));
+}
+
+extern "C" int mv_add_rows(void* y, long ldy, const void* x, long ldx, int rows, int cols, int dtype, hipStream_t stream) {
+    MV_REQUIRE(rows >= 0 && cols > 0 && ldy >= cols && ldx >= cols && y && x, "add_rows: bad sizes rows=%d cols=%d", rows, cols);
+    const long total = (long)rows * cols;
+    if (total == 0) return 0;
+    MV_DISPATCH_T(dtype, "add_rows",
+                  hipLaunchKernelGGL(add_rows_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (T*)y, ldy,
+                                     (const T*)x, ldx, cols, total));
+    return mv_check_launch("add_rows");
 }
 
 // float rows in place: x <- x * factor

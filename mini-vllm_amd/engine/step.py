@@ -126,6 +126,9 @@ class StepContext:
         self.page_size = 0
         # rows that a position encoding had gathered for this step (PositionEncoding.step_gather), by part
         self.position_rows: Dict[object, torch.Tensor] = {}
+        # what a part leaves for parts of later calls of the same step, by a key of their own choosing (the
+        # values a layer projected, which later layers blend into theirs)
+        self.carry: Dict[str, torch.Tensor] = {}
 
     def kv(self, call: int) -> KVView:
         try:

@@ -44,10 +44,22 @@ _SIGNATURES = {
     "mv_gemm_ref": (c_int, [c_void_p, c_long, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_int,
                             c_int, c_int, c_int, c_void_p]),
     # q, q_stride, out, out_stride, k_pages, v_pages, block_table, bt_width, page_size, positions, token_seq, n, H, Hkv, D,
-    # scale, window, first, gate, gate_stride, dtype, stream
+    # Dv, scale, window, first, gate, gate_stride, dtype, stream
     "mv_attention_ref": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
-                                 c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_long,
+                                 c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_long,
                                  c_int, c_void_p]),
+    # qkv, stride, q_off, k_off, v_off, positions, token_seq, block_table, bt_width, page_size, k_pages, v_pages, n, H, Hkv, D,
+    # Dv, q_weight, k_weight, weight_dtype, unit_norm, eps, table, rot_dim, interleaved, mix_rows, mix_stride, mix_weight,
+    # mix_weight_dtype, dtype, stream
+    "mv_qkv_rotate_norm_store": (c_int, [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                         c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int,
+                                         c_float, c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p]),
+    # lanes, plane, first, S, n, W, y, ldy, w_mix, w_out, w_in, w_norm, norm_dtype, eps, h, ldh, total, dtype, stream
+    "mv_hyper_step": (c_int, [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p,
+                              c_void_p, c_int, c_float, c_void_p, c_long, c_void_p, c_int, c_void_p]),
+    # tokens, table, rows, n, E, top, dense, ld_dense, ids, weights, stream
+    "mv_moe_table_route": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
+                                   c_void_p]),
     # resid, x, ldx, delta, weight, weight_dtype, eps, groups, out, ldo, rows, n_out, h, dtype, stream
     "mv_group_norm_rows": (c_int, [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_float, c_int, c_void_p, c_long,
                                    c_void_p, c_int, c_int, c_int, c_void_p]),
@@ -98,9 +110,9 @@ _SIGNATURES = {
 
 # entry points that only the bfloat16 library has
 _OPTIONAL_SIGNATURES = {
-    # x, ldx, ldx_head, w, n, H, IN, OUT, y, ldy, ldy_head, tail, table, positions, gate, ldg, token_seq, mode, stream
+    # x, ldx, ldx_head, w, n, H, IN, OUT, y, ldy, ldy_head, tail, table, positions, gate, ldg, gate_per_head, token_seq, mode, stream
     "mv_head_linear_mfma": (c_int, [c_void_p, c_long, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_long, c_int, c_int,
-                                    c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p]),
+                                    c_void_p, c_void_p, c_void_p, c_long, c_int, c_void_p, c_int, c_void_p]),
     # q, ldq, out, ldo, pages, pages_t, block_table, bt_width, page_size, positions, token_seq, n, H, R, DR, scale, stream
     "mv_attention_latent_mfma": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                          c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p]),
@@ -203,7 +215,7 @@ _OPTIONAL_SIGNATURES = {
     # x, ldx, ldx_head, w, weight_dtype, n, H, IN, OUT, y, ldy, ldy_head, tail, table, positions, gate, ldg, token_seq, mode,
     # dtype, stream
     "mv_head_linear": (c_int, [c_void_p, c_long, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_long, c_int,
-                               c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p]),
+                               c_int, c_void_p, c_void_p, c_void_p, c_long, c_int, c_void_p, c_int, c_int, c_void_p]),
     # q, ldq, out, ldo, pages, block_table, bt_width, page_size, positions, token_seq, n, H, R, DR, scale, dtype, stream
     "mv_attention_latent": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p,
                                     c_int, c_int, c_int, c_int, c_float, c_int, c_void_p]),
@@ -216,12 +228,14 @@ _OPTIONAL_SIGNATURES = {
     "mv_moe_route": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p,
                              c_void_p, c_void_p, c_void_p]),
     # gate_up, ld, dense, ld_dense, n, E, F, act, limit, slope, dtype, stream
-    "mv_moe_swiglu_scale": (c_int, [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_float, c_float, c_int,
-                                    c_void_p]),
+    "mv_moe_swiglu_scale": (c_int, [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_float, c_float,
+                                    c_int, c_void_p]),
     # y, ldy, h, ldh, dense, ld_dense, first, count, n, width, set, dtype, stream
     "mv_moe_identity_add": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_void_p]),
     "mv_scale_f32": (c_int, [c_void_p, c_long, c_int, c_int, c_float, c_void_p]),
+    # y, ldy, x, ldx, rows, cols, dtype, stream
+    "mv_add_rows": (c_int, [c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_void_p]),
     "mv_launch_empty": (c_int, [c_int, c_int, c_void_p, c_void_p]),
 }
 

@@ -904,8 +904,10 @@ class Ops:
 
     def head_linear(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, token_seq: torch.Tensor, tail: int = 0,
                     table: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
-                    gate: Optional[torch.Tensor] = None, w_rows: Optional[torch.Tensor] = None) -> None:
-        """Per head h: out[t, h, :OUT] = x[t, h, :IN] @ w[h] with w [heads, IN, OUT]. x [n, heads, IN + tail] in the
+                    gate: Optional[torch.Tensor] = None, w_rows: Optional[torch.Tensor] = None,
+                    gate_per_head: bool = False) -> None:
+        """Per head h: out[t, h, :OUT] = x[t, h, :IN] @ w[h] with w [heads, IN, OUT]. (With ``gate_per_head`` the gate is
+        [n, >= heads] rows, one number for all outputs of a head.) x [n, heads, IN + tail] in the
         activation type gives out float32 [n, heads, OUT + tail], the ``tail`` last inputs copied behind the outputs
         and rotated by the row's position (``table`` as for ``latent_prepare``); x float32 [n, heads, IN] gives out
         [n, heads * OUT] in the activation type, multiplied by sigmoid(gate [n, heads * OUT]) when a gate is given.
@@ -934,8 +936,9 @@ class Ops:
             ldy, ldy_head = out.stride(0) if n > 1 else H * OUT, OUT
             if gate is not None:
                 self._act(gate, "output gate")
-                if tuple(gate.shape) != (n, H * OUT) or gate.stride(1) != 1:
-                    raise KernelLibraryError("head_linear: the gate must be [n, heads * OUT]")
+                if gate.dim() != 2 or gate.shape[0] != n or gate.stride(1) != 1 \
+                        or (gate.shape[1] < H if gate_per_head else gate.shape[1] != H * OUT):
+                    raise KernelLibraryError("head_linear: the gate must be [n, heads * OUT], or [n, >= heads] with one number a head")
         else:
             raise KernelLibraryError(f"head_linear: {x.dtype} -> {out.dtype} with these options is not served")
         if w_rows is not None and n > 64 and self.use_fast_kernels and w_rows.dtype == torch.bfloat16 \
@@ -945,14 +948,15 @@ class Ops:
                 raise KernelLibraryError(f"head_linear: the row layout of the weight must be [{H}, {OUT}, {IN}]")
             if self.lib.offer("mv_head_linear_mfma", x.data_ptr(), x.stride(0), x.shape[2], w_rows.data_ptr(), n, H, IN, OUT,
                               out.data_ptr(), ldy, ldy_head, tail, _ptr(table), _ptr(positions), _ptr(gate),
-                              gate.stride(0) if gate is not None else 0, token_seq.data_ptr(), mode, self._stream()):
+                              gate.stride(0) if gate is not None else 0, int(gate_per_head), token_seq.data_ptr(), mode,
+                              self._stream()):
                 self._note("mv_head_linear_mfma", self._size(x, w, out), 2 * n * H * IN * OUT)
                 return
         self._note("mv_head_linear", self._size(x, w, out), 2 * n * H * IN * OUT)
         self.lib.call("mv_head_linear", x.data_ptr(), x.stride(0) if n > 1 else H * x.shape[2], x.shape[2], w.data_ptr(),
                       _weight_code(w, "head_linear weight"), n, H, IN, OUT, out.data_ptr(), ldy, ldy_head, tail, _ptr(table),
-                      _ptr(positions), _ptr(gate), (gate.stride(0) if n > 1 else H * OUT) if gate is not None else 0,
-                      token_seq.data_ptr(), mode, self.code, self._stream())
+                      _ptr(positions), _ptr(gate), (gate.stride(0) if n > 1 else gate.shape[1]) if gate is not None else 0,
+                      int(gate_per_head), token_seq.data_ptr(), mode, self.code, self._stream())
 
     def attention_latent(self, q: torch.Tensor, out: torch.Tensor, pages: torch.Tensor, block_table: torch.Tensor,
                          page_size: int, positions: torch.Tensor, token_seq: torch.Tensor, heads: int, kv_rank: int,
@@ -1050,20 +1054,41 @@ class Ops:
                       top, float(sum_eps), flags, dense.data_ptr(), ids.data_ptr(), weights.data_ptr(), self._stream())
 
     def moe_swiglu_scale(self, gate_up: torch.Tensor, dense: torch.Tensor, experts: int, ff: int, out: torch.Tensor,
-                         limit: float = 0.0, slope: float = 1.0) -> None:
+                         limit: float = 0.0, slope: float = 1.0, shared: int = 0) -> None:
         """out[t, e, c] = dense[t, e] * silu(gate_up[t, e*ff + c]) * gate_up[t, experts*ff + e*ff + c] (zero where the
         weight is zero, whatever the products hold). With ``limit`` > 0 the clamped pair instead: g = min(gate, limit),
-        u = clamp(up, -limit, limit), out = dense * g * sigmoid(slope * g) * (u + 1)."""
+        u = clamp(up, -limit, limit), out = dense * g * sigmoid(slope * g) * (u + 1). With ``shared`` > 0 the rows hold
+        that many gate and as many up columns of a shared expert behind the others', and out gets its pair, with the
+        weight one, behind the experts' columns."""
         self._act(gate_up, "gate_up"); self._act(out, "expert activations"); _dev(dense, "dense weights")
         n = gate_up.shape[0]
-        if tuple(gate_up.shape) != (n, 2 * experts * ff) or gate_up.stride(1) != 1 or tuple(out.shape) != (n, experts * ff) \
+        if tuple(gate_up.shape) != (n, 2 * experts * ff + 2 * shared) or gate_up.stride(1) != 1 \
+                or tuple(out.shape) != (n, experts * ff + shared) \
                 or not out.is_contiguous() or dense.dtype != torch.float32 or dense.shape[0] != n or dense.shape[1] < experts \
                 or dense.stride(1) != 1:
             raise KernelLibraryError("moe_swiglu_scale: operands do not fit")
         self._note("mv_moe_swiglu_scale", self._size(gate_up, out), 8 * out.numel())
-        self.lib.call("mv_moe_swiglu_scale", gate_up.data_ptr(), gate_up.stride(0) if n > 1 else 2 * experts * ff, dense.data_ptr(),
-                      dense.stride(0) if n > 1 else dense.shape[1], n, experts, ff, out.data_ptr(), float(limit), float(slope),
-                      self.code, self._stream())
+        self.lib.call("mv_moe_swiglu_scale", gate_up.data_ptr(), gate_up.stride(0) if n > 1 else gate_up.shape[1], dense.data_ptr(),
+                      dense.stride(0) if n > 1 else dense.shape[1], n, experts, ff, int(shared), out.data_ptr(), float(limit),
+                      float(slope), self.code, self._stream())
+
+    def moe_table_route(self, token_ids: torch.Tensor, table: torch.Tensor, experts: int, dense: torch.Tensor, ids: torch.Tensor,
+                        weights: torch.Tensor) -> None:
+        """Experts named by a table: row t uses table[token_ids[t]] (int32 [rows, top]), each with the weight 1 / top.
+        dense float32 [n, >= experts], ids int32 / weights float32 [n, top] are left as ``moe_route`` leaves them."""
+        n, top = ids.shape
+        for t, name in ((token_ids, "token ids"), (table, "expert table"), (ids, "ids")):
+            _dev(t, name)
+            if t.dtype != torch.int32 or not t.is_contiguous():
+                raise KernelLibraryError(f"moe_table_route: {name} must be contiguous int32")
+        _dev(dense, "dense weights"); _dev(weights, "weights")
+        if token_ids.numel() < n or table.dim() != 2 or table.shape[1] != top or dense.dtype != torch.float32 or dense.dim() != 2 \
+                or dense.shape[0] != n or dense.shape[1] < experts or dense.stride(1) != 1 or weights.dtype != torch.float32 \
+                or tuple(weights.shape) != (n, top) or not weights.is_contiguous():
+            raise KernelLibraryError("moe_table_route: operands do not fit")
+        self._note("mv_moe_table_route", self._size(dense, ids, weights) + n * (top + 1) * 4, n * experts)
+        self.lib.call("mv_moe_table_route", token_ids.data_ptr(), table.data_ptr(), table.shape[0], n, experts, top, dense.data_ptr(),
+                      dense.stride(0) if n > 1 else dense.shape[1], ids.data_ptr(), weights.data_ptr(), self._stream())
 
     def moe_identity_add(self, y: torch.Tensor, h: torch.Tensor, dense: torch.Tensor, first: int, count: int,
                          overwrite: bool = False) -> None:
@@ -1113,6 +1138,123 @@ class Ops:
         self._note("mv_moe_grouped", self._size(x, y) + used * 3 * ff * hidden * 2 + self._size(act, out) * 2,
                    2 * n * top * 3 * ff * hidden)
         return True
+
+    def hyper_step(self, lanes: torch.Tensor, out: Optional[torch.Tensor] = None, first: Optional[torch.Tensor] = None,
+                   write=None, read=None, total: Optional[torch.Tensor] = None) -> None:
+        """Several residual streams, float32 ``lanes`` [S, n, W]. ``write`` = (y [n, W] of the activation type, mix float32
+        [S, S] indexed [from, to], out_weights float32 [S]): lane t <- sum_s mix[s, t] lane s + out_weights[t] y, all from
+        the old lanes. ``read`` = (in_weights float32 [S], norm weight [W], eps): ``out`` [n, W] (activation type) =
+        rmsnorm(sum_s in_weights[s] lane s) * weight, from the lanes as the write leaves them. ``first`` float32 [n, W]:
+        the lanes do not exist yet, every one of them is this row. ``total`` float32 [n, W] gets the sum of the lanes
+        (behind a write without a read the lanes themselves are then not stored)."""
+        _dev(lanes, "residual lanes")
+        if lanes.dtype != torch.float32 or lanes.dim() != 3 or lanes.stride(2) != 1 or lanes.stride(1) != lanes.shape[2]:
+            raise KernelLibraryError("hyper_step: the lanes must be float32 [streams, n, width] with contiguous rows")
+        S, n, W = lanes.shape
+        for t, name in ((first, "first rows"), (total, "summed rows")):
+            if t is not None:
+                _dev(t, name)
+                if t.dtype != torch.float32 or tuple(t.shape) != (n, W) or not t.is_contiguous():
+                    raise KernelLibraryError(f"hyper_step: the {name} must be contiguous float32 [{n}, {W}]")
+        y = w_mix = w_out = w_in = w_norm = None
+        eps = 1.0
+        if write is not None:
+            y, w_mix, w_out = write
+            self._act(y, "sublayer output")
+            if y.dim() != 2 or y.shape[0] != n or y.shape[1] < W or y.stride(1) != 1:
+                raise KernelLibraryError(f"hyper_step: the sublayer output must be [{n}, {W}]")
+            for t, shape in ((w_mix, (S, S)), (w_out, (S,))):
+                _dev(t, "stream weights")
+                if t.dtype != torch.float32 or tuple(t.shape) != shape or not t.is_contiguous():
+                    raise KernelLibraryError(f"hyper_step: stream weights must be contiguous float32 {shape}")
+        if read is not None:
+            w_in, w_norm, eps = read
+            _dev(w_in, "stream weights"); _dev(w_norm, "norm weight")
+            if w_in.dtype != torch.float32 or tuple(w_in.shape) != (S,) or not w_in.is_contiguous() or w_norm.numel() != W \
+                    or not w_norm.is_contiguous():
+                raise KernelLibraryError(f"hyper_step: the read needs float32 [{S}] stream weights and a norm weight of {W}")
+            self._act(out, "normed rows")
+            if tuple(out.shape) != (n, W) or out.stride(1) != 1:
+                raise KernelLibraryError(f"hyper_step: the normed rows must be [{n}, {W}]")
+        if n == 0:
+            return
+        moved = (S if first is None else 1) + (S if (read is not None or total is None) else 0) + (1 if total is not None else 0)
+        self._note("mv_hyper_step", n * W * (4 * moved + (y.element_size() if y is not None else 0)
+                                               + (out.element_size() if read is not None else 0)), n * W * (2 * S * S + 2 * S + 4))
+        self.lib.call("mv_hyper_step", lanes.data_ptr(), lanes.stride(0), _ptr(first), S, n, W, _ptr(y),
+                      (y.stride(0) if n > 1 else y.shape[1]) if y is not None else 0, _ptr(w_mix), _ptr(w_out), _ptr(w_in),
+                      _ptr(w_norm), _weight_code(w_norm, "norm weight") if w_norm is not None else DTYPE_F32, float(eps),
+                      _ptr(out) if read is not None else 0, (out.stride(0) if n > 1 else W) if read is not None else 0,
+                      _ptr(total), self.code, self._stream())
+
+    def qkv_rotate_norm_store(self, qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+                              positions: torch.Tensor, token_seq: torch.Tensor, rope_table: Optional[torch.Tensor],
+                              interleaved: bool, unit_norm: bool, eps: float, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                              block_table: torch.Tensor, page_size: int, q_weight: Optional[torch.Tensor] = None,
+                              k_weight: Optional[torch.Tensor] = None, mix_rows: Optional[torch.Tensor] = None,
+                              mix_weight: Optional[torch.Tensor] = None) -> None:
+        """On the rows ``qkv`` = [q | k | v | ...] of a step: q and k heads are rotated over their first channels by the
+        row's position (``rope_table`` float32 [positions, rot] = cat(cos, sin)) and, with ``unit_norm``, divided by their
+        root mean square afterwards (times ``q_weight`` / ``k_weight`` where given); q stays in the rows, k goes to the key
+        pages [pages, kv_heads, page_size, head_dim]. The values go to the value pages [pages, kv_heads, value_dim,
+        page_size]; with ``mix_rows`` [n, >= kv_heads * value_dim] and ``mix_weight`` (one number on the device, m) they
+        are (1 - m) v + m mix_rows first."""
+        self._act(qkv, "qkv"); self._act(k_pages, "key pages"); self._act(v_pages, "value pages")
+        n = qkv.shape[0]
+        q_dim, kv_dim, v_dim = num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * value_dim
+        if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < q_dim + kv_dim + v_dim:
+            raise KernelLibraryError(f"qkv_rotate_norm_store: rows {tuple(qkv.shape)} do not hold {q_dim + kv_dim + v_dim} columns")
+        if tuple(k_pages.shape[1:]) != (num_kv_heads, page_size, head_dim) or tuple(v_pages.shape[1:]) != (num_kv_heads, value_dim, page_size) \
+                or not k_pages.is_contiguous() or not v_pages.is_contiguous():
+            raise KernelLibraryError(f"qkv_rotate_norm_store: pages {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not match "
+                                     f"[pages, {num_kv_heads}, {page_size}, {head_dim}] / [pages, {num_kv_heads}, {value_dim}, {page_size}]")
+        self._ints(n, positions=(positions, n), token_seq=(token_seq, n))
+        _dev(block_table, "block table")
+        if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+            raise KernelLibraryError("qkv_rotate_norm_store: the block table must be a contiguous int32 matrix")
+        rot = 0
+        if rope_table is not None:
+            _dev(rope_table, "rope table")
+            if rope_table.dtype != torch.float32 or rope_table.dim() != 2 or not rope_table.is_contiguous() \
+                    or rope_table.shape[1] > head_dim or rope_table.shape[1] % 2:
+                raise KernelLibraryError("qkv_rotate_norm_store: the rope table must be contiguous float32 [positions, rot <= head_dim]")
+            rot = rope_table.shape[1]
+        wcode = DTYPE_F32
+        if (q_weight is None) != (k_weight is None):
+            raise KernelLibraryError("qkv_rotate_norm_store: norm weights come in pairs")
+        if q_weight is not None:
+            wcode = _weight_code(q_weight, "q norm weight")
+            if q_weight.numel() != head_dim or k_weight.numel() != head_dim or k_weight.dtype != q_weight.dtype:
+                raise KernelLibraryError("qkv_rotate_norm_store: norm weights must both hold head_dim elements")
+        mcode, mstride = DTYPE_F32, 0
+        if mix_rows is not None:
+            self._act(mix_rows, "rows blended into the values"); _dev(mix_weight, "blend weight")
+            if mix_rows.dim() != 2 or mix_rows.shape[0] != n or mix_rows.shape[1] < v_dim or mix_rows.stride(1) != 1 \
+                    or mix_weight is None or mix_weight.numel() != 1:
+                raise KernelLibraryError(f"qkv_rotate_norm_store: blending needs rows [{n}, >= {v_dim}] and one weight")
+            mcode = _weight_code(mix_weight, "blend weight")
+            mstride = mix_rows.stride(0) if n > 1 else mix_rows.shape[1]
+        if n == 0:
+            return
+        self._note("mv_qkv_rotate_norm_store", n * (2 * q_dim + 2 * kv_dim + (3 if mix_rows is not None else 2) * v_dim) * qkv.element_size()
+                   + n * rot * 4, 10 * n * (q_dim + kv_dim))
+        self.lib.call("mv_qkv_rotate_norm_store", qkv.data_ptr(), qkv.stride(0) if n > 1 else qkv.shape[1], 0, q_dim, q_dim + kv_dim,
+                      positions.data_ptr(), token_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
+                      k_pages.data_ptr(), v_pages.data_ptr(), n, num_heads, num_kv_heads, head_dim, value_dim, _ptr(q_weight),
+                      _ptr(k_weight), wcode, int(unit_norm), float(eps), _ptr(rope_table), rot, int(interleaved), _ptr(mix_rows),
+                      mstride, _ptr(mix_weight), mcode, self.code, self._stream())
+
+    def add_rows(self, y: torch.Tensor, x: torch.Tensor) -> None:
+        """In place on rows of the activation type: y <- y + x (added in float32, rounded once)."""
+        self._act(y, "rows"); self._act(x, "rows to add")
+        if y.dim() != 2 or tuple(x.shape) != tuple(y.shape) or y.stride(1) != 1 or x.stride(1) != 1:
+            raise KernelLibraryError("add_rows: two matrices of one shape with contiguous rows are needed")
+        rows, cols = y.shape
+        if rows == 0:
+            return
+        self._note("mv_add_rows", 3 * self._size(y), rows * cols)
+        self.lib.call("mv_add_rows", y.data_ptr(), y.stride(0) if rows > 1 else cols, x.data_ptr(), x.stride(0) if rows > 1 else cols,
+                      rows, cols, self.code, self._stream())
 
     def scale_f32(self, x: torch.Tensor, factor: float) -> None:
         """In place on float32 [rows, cols]: x <- x * factor."""
@@ -1731,10 +1873,12 @@ class Ops:
     def attention(self, q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                   block_table: torch.Tensor, page_size: int, positions: torch.Tensor, token_seq: torch.Tensor,
                   num_heads: int, num_kv_heads: int, head_dim: int, scale: float, window: Optional[int],
-                  plan: Optional["AttentionPlan"] = None, keep_first: int = 0, gate: Optional[torch.Tensor] = None) -> None:
+                  plan: Optional["AttentionPlan"] = None, keep_first: int = 0, gate: Optional[torch.Tensor] = None,
+                  value_dim: Optional[int] = None) -> None:
         """Causal attention of the step's queries over the paged cache.
 
-        q: [n, >= H*D] rows (a view into the qkv rows), out: [n, H*D]. The query at position p
+        q: [n, >= H*D] rows (a view into the qkv rows), out: [n, H*Dv] (``value_dim`` Dv: the size of a value row
+        where it differs from a key's; such sizes take the general kernel). The query at position p
         of sequence s sees keys max(0, p - window) .. p of s and, with ``keep_first``, the first
         ``keep_first`` positions of s however far back they lie. ``gate`` [n, >= H] (a view into the
         packed rows): head h's output is multiplied by sigmoid(gate[:, h]). ``plan`` carries what the faster
@@ -1743,12 +1887,13 @@ class Ops:
         self._act(q, "queries"); self._act(out, "attention output")
         self._act(k_pages, "key pages"); self._act(v_pages, "value pages")
         n = q.shape[0]
-        hd = num_heads * head_dim
-        if q.dim() != 2 or q.shape[1] < hd or q.stride(1) != 1 or out.shape != (n, hd) or out.stride(1) != 1:
+        vdim = head_dim if value_dim is None else int(value_dim)
+        hd = num_heads * vdim
+        if q.dim() != 2 or q.shape[1] < num_heads * head_dim or q.stride(1) != 1 or out.shape != (n, hd) or out.stride(1) != 1:
             raise KernelLibraryError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not hold "
-                                     f"{num_heads} heads of {head_dim}")
+                                     f"{num_heads} heads of {head_dim} / {vdim}")
         if tuple(k_pages.shape[1:]) != (num_kv_heads, page_size, head_dim) or \
-                tuple(v_pages.shape[1:]) != (num_kv_heads, head_dim, page_size) or \
+                tuple(v_pages.shape[1:]) != (num_kv_heads, vdim, page_size) or \
                 not k_pages.is_contiguous() or not v_pages.is_contiguous():
             raise KernelLibraryError(f"attention: pages {tuple(k_pages.shape)} / {tuple(v_pages.shape)} have the "
                                      f"wrong layout for {num_kv_heads} heads of {head_dim}, page {page_size}")
@@ -1773,13 +1918,13 @@ class Ops:
             if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < num_heads or gate.stride(1) != 1:
                 raise KernelLibraryError(f"attention: gates {tuple(gate.shape)} do not hold {num_heads} numbers a row")
             gs = gate.stride(0) if n > 1 else gate.shape[1]
-        if self._attention_fast(q, qs, out, os_, k_pages, v_pages, block_table, page_size, positions, token_seq,
-                                num_heads, num_kv_heads, head_dim, scale, w, plan, first, gate, gs):
+        if vdim == head_dim and self._attention_fast(q, qs, out, os_, k_pages, v_pages, block_table, page_size, positions,
+                                                     token_seq, num_heads, num_kv_heads, head_dim, scale, w, plan, first, gate, gs):
             return
         self._note_attention("mv_attention_ref", plan, n, num_heads, num_kv_heads, head_dim, q.element_size())
         self.lib.call("mv_attention_ref", q.data_ptr(), qs, out.data_ptr(), os_, k_pages.data_ptr(),
                       v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], page_size,
-                      positions.data_ptr(), token_seq.data_ptr(), n, num_heads, num_kv_heads, head_dim,
+                      positions.data_ptr(), token_seq.data_ptr(), n, num_heads, num_kv_heads, head_dim, vdim,
                       float(scale), w, first, _ptr(gate), gs, self.code, self._stream())
 
     def _note_attention(self, entry: str, plan, n_tokens: int, H: int, Hkv: int, D: int, item: int, splits: int = 1) -> None:

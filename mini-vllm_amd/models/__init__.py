@@ -4,4 +4,5 @@ from . import qwen3  # registers "Qwen3ForCausalLM"
 from . import bolapel  # registers "Bolapel"
 from . import dutilix  # registers "Dutilix"
 from . import zedudra  # registers "Zedudra"
+from . import furanex  # registers "Furanex"
 from .causal_lm import CausalLM, expected_tensors

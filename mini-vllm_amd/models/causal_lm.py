@@ -180,6 +180,7 @@ class CausalLM:
         resid = rt.workspace.get("resid", (n, plan.hidden_size), torch.float32)
         # what position encodings want gathered for the whole step rides on the first kernel
         ctx.position_rows = {}
+        ctx.carry = {}
         gathers = [job for job in (part.step_gather(ctx) for part in self.position_parts.values()
                                    if hasattr(part, "step_gather")) if job is not None]
         if gathers and getattr(self.embedding, "carries_gather", False):
@@ -199,6 +200,9 @@ class CausalLM:
                 block.forward(stream, ctx, call_index, next_norm=after.entry_norm(), next_part=after.entry_part())
             else:
                 block.forward(stream, ctx, call_index)
+        closer = getattr(self.blocks[plan.calls[-1].layer], "close_stream", None)
+        if closer is not None:
+            closer(stream, ctx)      # an arrangement that keeps the residual in another form brings ``resid`` up to date
         m = ctx.n_logit_rows
         if m == 0:
             discard = getattr(stream.delta, "discard", None)

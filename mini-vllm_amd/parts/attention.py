@@ -18,6 +18,13 @@ number per head, read from the same packed product as q, k and v; ``keep_first``
 query also sees the sequence's first ``keep_first`` positions however far back they lie, at their true
 positions; ``value_from_key``: there is no value projection, the values are the keys as projected,
 before norm and rotation. Softmax weighting with any of the last three runs ``_forward_kept``.
+
+``unit_norm_after_rotation``: q and k are rotated first and then divided by their root mean square per head
+(x / sqrt(mean(x^2) + qk_norm_eps), no weight). ``value_mix``: values are shared between layers of a model
+within a token: a layer with ``value_mix = "source"`` leaves the values it projected for the step's tokens in
+``ctx.carry[value_mix_key]``; a layer with ``"blend"`` caches (1 - m) v + m v_source instead of its own v,
+with m its stored number ``value_mix`` (both must have the same kv heads and value size). Softmax weighting
+with either of these, or with values of another size than keys, runs ``_forward_rotated``.
 """
 from __future__ import annotations
 
@@ -55,6 +62,9 @@ class AttentionSpec(PartSpec):
     cache_keeps_all: bool = False
     keep_first: int = 0                      # with a window: the sequence's first positions stay visible
     value_from_key: bool = False             # values = keys as projected (no value projection)
+    unit_norm_after_rotation: bool = False   # q, k <- x / rms(x) per head, behind the rotation, without a weight
+    value_mix: Optional[str] = None          # "source" or "blend", see above
+    value_mix_key: str = ""
 
     @property
     def q_dim(self) -> int:
@@ -80,13 +90,23 @@ class AttentionSpec(PartSpec):
     def plain(self) -> bool:
         """The reference's layer: softmax over all keys or a window, values as large as keys."""
         return (self.weighting == "softmax" and self.chunk is None and self.value_dim in (None, self.head_dim)
-                and not self.head_gate and not self.score_bias and not self.keep_first and not self.value_from_key)
+                and not self.head_gate and not self.score_bias and not self.keep_first and not self.value_from_key
+                and not self.unit_norm_after_rotation and self.value_mix is None)
+
+    @property
+    def rotated(self) -> bool:
+        """Softmax with the unit norm behind the rotation, values shared between layers, or values of a size of their own."""
+        return (self.weighting == "softmax" and self.chunk is None and not self.score_bias and not self.bias
+                and not self.qk_norm and not self.head_gate and not self.keep_first and not self.value_from_key
+                and not self.shares_kv
+                and (self.unit_norm_after_rotation or self.value_mix is not None or self.value_dim not in (None, self.head_dim)))
 
     @property
     def kept(self) -> bool:
         """Softmax over a window (or all keys) with kept first positions, head gates or values taken from the keys."""
         return (self.weighting == "softmax" and self.chunk is None and self.value_dim in (None, self.head_dim)
-                and not self.score_bias and not self.bias and not self.qk_norm and not self.plain)
+                and not self.score_bias and not self.bias and not self.qk_norm and not self.plain and not self.rotated
+                and not self.unit_norm_after_rotation and self.value_mix is None)
 
 
 @register_mixer(AttentionSpec.kind)
@@ -106,6 +126,8 @@ class Attention(Mixer):
             t["score_bias"] = TensorDecl((spec.num_heads,), init="zeros_normal")
         if spec.head_gate:
             t["head_gate"] = TensorDecl((spec.num_heads, spec.hidden_size))
+        if spec.value_mix == "blend":
+            t["value_mix"] = TensorDecl((), init="zeros_normal")
         if spec.bias:
             t["q_bias"] = TensorDecl((spec.q_dim,), init="zeros_normal")
             t["o_bias"] = TensorDecl((spec.hidden_size,), init="zeros_normal")
@@ -141,7 +163,12 @@ class Attention(Mixer):
             raise ValueError(f"{spec.num_heads} query heads are not a multiple of {spec.num_kv_heads} kv heads")
         if spec.weighting not in ("softmax", "sigmoid"):
             raise ValueError(f"attention weighting must be 'softmax' or 'sigmoid', got {spec.weighting!r}")
-        if not spec.plain and not spec.kept and (spec.weighting != "sigmoid" or spec.bias):
+        if spec.value_mix not in (None, "source", "blend") or (spec.value_mix and not spec.value_mix_key):
+            raise ValueError(f"value_mix must be None, 'source' or 'blend' with a key, got {spec.value_mix!r}, {spec.value_mix_key!r}")
+        if (spec.unit_norm_after_rotation or spec.value_mix) and not spec.rotated:
+            raise NotImplementedError("the unit norm behind the rotation and values shared between layers are built for softmax "
+                                      "weighting over all keys or a window, without biases, weighted q/k norms, gates or a shared cache")
+        if not spec.plain and not spec.kept and not spec.rotated and (spec.weighting != "sigmoid" or spec.bias):
             raise NotImplementedError("chunks, a value size of its own and a score bias are built for sigmoid weighting "
                                       "without projection biases; kept first positions, head gates and values taken from "
                                       "the keys also for softmax weighting without biases and query/key norms")
@@ -167,6 +194,7 @@ class Attention(Mixer):
         self.w_o = tensors["o"]
         self.q_norm = tensors.get("q_norm")
         self.k_norm = tensors.get("k_norm")
+        self.value_mix = tensors.get("value_mix")
         self.position = position
         self.rotary = position.rotary() if position is not None else None
         if position is not None and self.rotary is None and not hasattr(position, "apply"):
@@ -192,6 +220,8 @@ class Attention(Mixer):
 
     def forward(self, x: torch.Tensor, ctx, call: int, fold=None) -> torch.Tensor:
         spec, rt, ops = self.spec, self.rt, self.rt.ops
+        if spec.rotated:
+            return self._forward_rotated(x, ctx, call)
         if spec.kept:
             return self._forward_kept(x, ctx, call)
         if not spec.plain:
@@ -282,5 +312,38 @@ class Attention(Mixer):
         ops.attention(packed[:, :spec.q_dim], attn, kv.k_pages, kv.v_pages, kv.block_table, kv.page_size, ctx.positions,
                       ctx.token_seq, spec.num_heads, spec.num_kv_heads, spec.head_dim, spec.scale, spec.window,
                       plan=ctx.attention_plan, keep_first=spec.keep_first, gate=gate)
+        y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
+        return ops.gemm(attn, self.w_o, y, defer_sum=True) or y
+
+    def _forward_rotated(self, x: torch.Tensor, ctx, call: int) -> torch.Tensor:
+        """Softmax weighting with the unit norm behind the rotation, values blended with another layer's, values of any size."""
+        spec, rt, ops, ws = self.spec, self.rt, self.rt.ops, self.rt.workspace
+        if not isinstance(x, torch.Tensor):
+            x = x.materialize()
+        n = x.shape[0]
+        # the layer whose values the later ones blend in keeps its rows in a buffer of its own for the rest of the step
+        name = f"attn.qkv.{spec.value_mix_key}" if spec.value_mix == "source" else "attn.qkv"
+        packed = ws.get(name, (n, self.width), rt.dtype)
+        ops.gemm(x, self.w_qkv, packed)
+        kv = ctx.kv(call)
+        table, interleaved = (self.rotary if self.rotary is not None else (None, False))
+        if self.position is not None and self.rotary is None:
+            raise NotImplementedError("this attention takes its rotation from a rotary table")
+        v_off = spec.q_dim + spec.kv_dim
+        mix_rows = None
+        if spec.value_mix == "source":
+            ctx.carry[spec.value_mix_key] = packed[:, v_off:v_off + spec.v_dim]
+        elif spec.value_mix == "blend":
+            mix_rows = ctx.carry.get(spec.value_mix_key)
+            if mix_rows is None or mix_rows.shape[0] != n or mix_rows.shape[1] != spec.v_dim:
+                raise RuntimeError(f"no layer in front of this one left values of {spec.v_dim} columns under {spec.value_mix_key!r}")
+        ops.qkv_rotate_norm_store(packed, spec.num_heads, spec.num_kv_heads, spec.head_dim, spec.v_head_dim, ctx.positions,
+                                  ctx.token_seq, table, interleaved, spec.unit_norm_after_rotation, spec.qk_norm_eps,
+                                  kv.k_pages, kv.v_pages, kv.block_table, kv.page_size, mix_rows=mix_rows,
+                                  mix_weight=self.value_mix if mix_rows is not None else None)
+        attn = ws.get("attn.out", (n, spec.out_dim), rt.dtype)
+        ops.attention(packed[:, :spec.q_dim], attn, kv.k_pages, kv.v_pages, kv.block_table, kv.page_size, ctx.positions,
+                      ctx.token_seq, spec.num_heads, spec.num_kv_heads, spec.head_dim, spec.scale, spec.window,
+                      plan=ctx.attention_plan, value_dim=spec.v_head_dim)
         y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
         return ops.gemm(attn, self.w_o, y, defer_sum=True) or y

@@ -344,7 +344,7 @@ class HiddenStream:
     defer_sum=True)`` returned in its place (an output whose partial sums the norm's kernel adds
     up itself; it has ``shape``, ``materialize()`` and ``discard()``)."""
 
-    __slots__ = ("resid", "delta", "spare", "weighted", "normed")
+    __slots__ = ("resid", "delta", "spare", "weighted", "normed", "lanes", "lanes_write")
 
     def __init__(self, resid: torch.Tensor, spare: Optional[torch.Tensor] = None):
         self.resid = resid
@@ -359,6 +359,12 @@ class HiddenStream:
         # a second buffer of the same shape: a kernel that adds the delta while other workgroups
         # still read the old sum writes the new sum here, and the two change places
         self.spare = spare
+        # a block arrangement that keeps several residual streams holds them here, float32 [streams, tokens,
+        # hidden], together with the last sublayer's output that has not been written into them yet; while
+        # they exist ``resid`` is stale, and the arrangement brings it up to date when it hands the stream
+        # to a block of another kind or to the model's last norm
+        self.lanes = None
+        self.lanes_write = None
 
 
 class PendingNorm:

@@ -249,3 +249,103 @@ class TokenShiftEntry:
 
     def __init__(self, mix: torch.Tensor):
         self.mix = mix
+
+
+@dataclass(frozen=True)
+class HyperConnectionBlockSpec(PartSpec):
+    """Pre-norm sublayers on ``streams`` residual streams of width ``hidden_size`` instead of one."""
+    kind = "hyper_connections"
+    hidden_size: int = 0
+    streams: int = 1
+    has_ffn: bool = True            # a layer without a feed-forward has no second set of stream weights
+
+
+class HyperEntry:
+    """What a block on several residual streams offers the block in front of it: its first sublayer's read,
+    so that a block of the same kind can leave its last write to that read's kernel."""
+
+    def __init__(self, block: "HyperConnectionBlock"):
+        self.block = block
+
+
+@register_block(HyperConnectionBlockSpec.kind)
+class HyperConnectionBlock(Block):
+    """A token's residual is S streams x_1 .. x_S, all equal to the embedding's output in front of the first
+    layer. Sublayer q (1: mixer, 2: feed-forward) with its stored weights ``hc<q>.in`` [S], ``hc<q>.out`` [S]
+    and ``hc<q>.mix`` [S, S] (indexed [from, to]):
+
+        u = sum_s in[s] x_s;   y = sublayer(norm_q(u));   x_t <- sum_s mix[s, t] x_s + out[t] y   (all t at once)
+
+    Behind the last layer the streams are summed into the plain residual. The streams live in
+    ``HiddenStream.lanes`` (float32); a write waits in ``lanes_write`` for the kernel of the next read, so
+    the streams are read and written once between two sublayers (``ops.hyper_step``). The norms must be
+    plain scaled RMS norms: the read's kernel applies them itself."""
+    norm_slots: Tuple[str, ...] = ("norm1", "norm2")
+    accepts_next_norm = True
+    wants_runtime = True
+
+    @classmethod
+    def slots_for(cls, has_ffn: bool) -> Tuple[str, ...]:
+        return cls.norm_slots if has_ffn else cls.norm_slots[:1]
+
+    @classmethod
+    def tensors(cls, spec: HyperConnectionBlockSpec):
+        from .base import TensorDecl
+        S = spec.streams
+        t = {}
+        for q in ((1, 2) if spec.has_ffn else (1,)):
+            t[f"hc{q}.in"] = TensorDecl((S,), init="ones_normal")
+            t[f"hc{q}.out"] = TensorDecl((S,), init="ones_normal")
+            t[f"hc{q}.mix"] = TensorDecl((S, S), init="identity_normal")
+        return t
+
+    def __init__(self, spec: HyperConnectionBlockSpec, norms: Dict[str, Norm], mixer: Mixer, ffn: FeedForward,
+                 tensors=None, rt=None):
+        if rt is None or tensors is None:
+            raise ValueError("a block on several residual streams needs its tensors and the runtime")
+        if spec.streams < 1 or spec.streams > 8:
+            raise ValueError(f"1 to 8 residual streams are served, got {spec.streams}")
+        self.spec, self.rt, self.mixer, self.ffn = spec, rt, mixer, ffn
+        self.sublayers = []
+        for q, part in ((1, mixer), (2, ffn)):
+            if part is None:
+                continue
+            form = norms[f"norm{q}"].as_scaled_rms()
+            if form is None or form[2]:
+                raise ValueError("the norms of a block on several residual streams must be plain scaled RMS norms")
+            # the residual sum is float32 whatever type the weights are stored in
+            w = {k: tensors[f"hc{q}.{k}"].to(torch.float32).contiguous() for k in ("in", "out", "mix")}
+            self.sublayers.append((part, w, form[0], form[1]))
+
+    def entry_norm(self) -> Optional[Norm]:
+        return None                     # the read applies it: no product may take it over
+
+    def entry_part(self):
+        return HyperEntry(self)
+
+    def forward(self, stream: HiddenStream, ctx, call: int, next_norm: Optional[Norm] = None, next_part=None) -> None:
+        rt, ops, spec = self.rt, self.rt.ops, self.spec
+        n = stream.resid.shape[0]
+        first = None
+        if stream.lanes is None:
+            if stream.delta is not None:
+                raise RuntimeError("a block on several residual streams cannot take a stream with a pending delta")
+            stream.lanes = rt.workspace.get("hyper.lanes", (spec.streams, n, spec.hidden_size), torch.float32)
+            first = stream.resid
+        for index, (part, w, norm_weight, eps) in enumerate(self.sublayers):
+            h = rt.workspace.get("normed", (n, spec.hidden_size), rt.dtype)
+            ops.hyper_step(stream.lanes, out=h, first=first, write=stream.lanes_write, read=(w["in"], norm_weight, eps))
+            first, stream.lanes_write = None, None
+            y = part.forward(h, ctx, call) if index == 0 and part is self.mixer else part.forward(h, ctx)
+            if not isinstance(y, torch.Tensor):
+                y = y.materialize()
+            stream.lanes_write = (y, w["mix"], w["out"])
+        if not isinstance(next_part, HyperEntry):
+            self.close_stream(stream, ctx)
+
+    def close_stream(self, stream: HiddenStream, ctx) -> None:
+        """The last write and the sum of the streams: ``stream.resid`` is the plain residual again."""
+        if stream.lanes is None:
+            return
+        self.rt.ops.hyper_step(stream.lanes, write=stream.lanes_write, total=stream.resid)
+        stream.lanes, stream.lanes_write, stream.delta = None, None, None

@@ -9,8 +9,13 @@ From the mixer's input h:
 
 Head h's key is [W_uk,h c | k_rot] and its value W_uv,h c; the score of query i and key j <= i is
 (q_plain . W_uk c_j + rot(q_rot) . k_rot,j) * scale, softmax over the visible keys. The heads'
-outputs are concatenated, multiplied by sigmoid(W_g h) when ``output_gate`` is set, and projected
-by W_o.
+outputs are concatenated, multiplied by sigmoid(W_g h) when ``output_gate`` is set (with ``head_gate`` W_g has
+one row a head and the whole head is multiplied by that one number), and projected by W_o.
+
+``rot_neighbours``: the rotation pairs channel 2i with 2i + 1 instead of i with i + rot_dim / 2. A score only sums
+products of a query's channel with the same channel of a key, so it does not change when the rotated channels of
+both are put in another order: the rows of W_uq and W_dkv that make them are reordered once, when the part is built
+(even channels first, then the odd ones), and the kernels rotate in half-split pairs as before.
 
 Only [c | k_rot] is cached, one row of ``kv_rank + rot_dim`` numbers per token, and c once more in
 the slot-contiguous layout that the MFMA kernel's second product reads (``LatentNeed``). Keys and values are never expanded: the query is carried into the latent's space
@@ -56,6 +61,8 @@ class LatentAttentionSpec(PartSpec):
     scale: float = 1.0
     norm_eps: float = 1e-6              # of the two latent norms
     output_gate: bool = False
+    head_gate: bool = False             # with output_gate: one gate a head instead of one a channel
+    rot_neighbours: bool = False        # the rotation pairs neighbouring channels
     position: Optional[PartSpec] = None     # a rotary encoding over rot_dim channels (None: rot_dim must be 0)
 
 
@@ -72,7 +79,7 @@ class LatentAttention(Mixer):
              "uk": TensorDecl((H * spec.plain_dim, spec.kv_rank)), "uv": TensorDecl((H * spec.value_dim, spec.kv_rank)),
              "o": TensorDecl((hid, H * spec.value_dim))}
         if spec.output_gate:
-            t["g"] = TensorDecl((H * spec.value_dim, hid))
+            t["g"] = TensorDecl((H if spec.head_gate else H * spec.value_dim, hid))
         return t
 
     @classmethod
@@ -90,10 +97,22 @@ class LatentAttention(Mixer):
                 raise ValueError("latent attention rotates its rot_dim channels in half-split pairs: it needs a rotary "
                                  "encoding over exactly rot_dim channels")
             self.table = rotary[0]
+        if spec.head_gate and not spec.output_gate:
+            raise ValueError("latent attention: head_gate says how the output gate is shaped; it needs output_gate")
         names = ["dq", "dkv"] + (["g"] if spec.output_gate else [])
         dtypes = {tensors[p].dtype for p in names}
         if len(dtypes) != 1:
             raise ValueError(f"latent attention: the projections are stored in different dtypes {dtypes}; cannot pack them")
+        tensors = dict(tensors)
+        if spec.rot_neighbours and spec.rot_dim:
+            # rotated channels in the order even, odd: pair (2i, 2i + 1) becomes (i, i + rot_dim / 2)
+            dr, dh = spec.rot_dim, spec.plain_dim + spec.rot_dim
+            order = torch.cat([torch.arange(0, dr, 2), torch.arange(1, dr, 2)]).to(tensors["dkv"].device)
+            rows = torch.cat([torch.arange(spec.kv_rank, device=order.device), spec.kv_rank + order])
+            tensors["dkv"] = tensors["dkv"].index_select(0, rows).contiguous()
+            head = torch.cat([torch.arange(spec.plain_dim, device=order.device), spec.plain_dim + order])
+            rows = (torch.arange(spec.num_heads, device=order.device)[:, None] * dh + head[None, :]).reshape(-1)
+            tensors["uq"] = tensors["uq"].index_select(0, rows).contiguous()
         blocks = [tensors[p] for p in names]
         self.gate_offset = spec.q_rank + spec.kv_rank + spec.rot_dim
         pad = (-sum(b.shape[0] for b in blocks)) % 8
@@ -131,7 +150,9 @@ class LatentAttention(Mixer):
         ops.attention_latent(qa, mixed, pages, kv.block_table, kv.page_size, ctx.positions, ctx.token_seq, H, R, dr,
                              spec.scale, plan=ctx.attention_plan, pages_t=pages_t)
         heads = ws.get("latent.heads", (n, H * spec.value_dim), rt.dtype)
-        gate = packed[:, self.gate_offset:self.gate_offset + H * spec.value_dim] if spec.output_gate else None
-        ops.head_linear(mixed, self.w_uv, heads, ctx.token_seq, gate=gate, w_rows=self.w_uv_rows)
+        gate = None
+        if spec.output_gate:
+            gate = packed[:, self.gate_offset:self.gate_offset + (H if spec.head_gate else H * spec.value_dim)]
+        ops.head_linear(mixed, self.w_uv, heads, ctx.token_seq, gate=gate, w_rows=self.w_uv_rows, gate_per_head=spec.head_gate)
         y = ws.get("mixer.out", (n, spec.hidden_size), rt.dtype)
         return ops.gemm(heads, self.w_o, y, defer_sum=True) or y

@@ -65,6 +65,12 @@ class RoutedExpertsSpec(PartSpec):
     activation: str = "swiglu"           # or "clamped" (with ``limit`` and ``gate_slope``)
     limit: float = 0.0
     gate_slope: float = 1.702
+    # "table": no router product; a stored integer table [table_rows, top] names the experts of every token id, each
+    # with the weight 1 / top (``groups``, ``correction``, ``scoring`` and ``normalize`` then mean nothing)
+    router: str = "learned"
+    table_rows: int = 0
+    # > 0: a shared expert of that width (a gated pair like the others) runs for every token and is added
+    shared_size: int = 0
 
     @property
     def router_outputs(self) -> int:
@@ -77,7 +83,14 @@ class RoutedExperts(FeedForward):
 
     @classmethod
     def tensors(cls, spec: RoutedExpertsSpec) -> Dict[str, TensorDecl]:
-        t = {"router": TensorDecl((spec.router_outputs, spec.hidden_size))}
+        if spec.router == "table":
+            t = {"table": TensorDecl((spec.table_rows, spec.top), init=f"distinct_below:{spec.num_experts}", integer=True)}
+        else:
+            t = {"router": TensorDecl((spec.router_outputs, spec.hidden_size))}
+        if spec.shared_size:
+            t["shared.gate"] = TensorDecl((spec.shared_size, spec.hidden_size))
+            t["shared.up"] = TensorDecl((spec.shared_size, spec.hidden_size))
+            t["shared.down"] = TensorDecl((spec.hidden_size, spec.shared_size))
         if spec.correction:
             t["correction"] = TensorDecl((spec.router_outputs,), init="zeros_normal")
         for e in range(spec.num_experts):
@@ -95,18 +108,41 @@ class RoutedExperts(FeedForward):
                 or spec.activation not in ("swiglu", "clamped") or (spec.activation == "clamped" and not spec.limit > 0):
             raise ValueError(f"routed experts: unknown scoring, group worth or activation, or a clamped pair without a "
                              f"positive limit: {spec}")
+        if spec.router not in ("learned", "table") or spec.shared_size < 0:
+            raise ValueError(f"routed experts: the router is 'learned' or 'table' and a shared expert's width >= 0: {spec}")
+        if spec.router == "table" and (spec.identity_experts or spec.correction or spec.table_rows < 1 or not spec.num_experts):
+            raise ValueError(f"routed experts: a table names experts with tensors, for every token id: {spec}")
+        if spec.shared_size and not spec.num_experts:
+            raise ValueError("routed experts: a shared expert stands beside experts with tensors")
         self.spec, self.rt = spec, rt
-        self.w_router = tensors["router"]
+        self.w_router = tensors.get("router")
+        self.table = tensors.get("table")
         self.correction = tensors.get("correction")
         n_e = spec.num_experts
         if n_e:
-            dtypes = {tensors[f"{k}.{e}"].dtype for e in range(n_e) for k in ("gate", "up", "down")}
+            names = [f"{k}.{e}" for e in range(n_e) for k in ("gate", "up", "down")]
+            if spec.shared_size:
+                names += ["shared.gate", "shared.up", "shared.down"]
+            dtypes = {tensors[name].dtype for name in names}
             if len(dtypes) != 1:
                 raise ValueError(f"routed experts: the experts are stored in different dtypes {dtypes}; cannot pack them")
-            # rows: every expert's gate block, then every expert's up block; the down matrices side by side
-            self.w_gate_up = torch.cat([tensors[f"gate.{e}"] for e in range(n_e)]
-                                       + [tensors[f"up.{e}"] for e in range(n_e)], dim=0).contiguous()
-            self.w_down = torch.cat([tensors[f"down.{e}"] for e in range(n_e)], dim=1).contiguous()
+            # rows: every expert's gate block, then every expert's up block; the down matrices side by side. A shared
+            # expert's gate and up rows come behind those and its down matrix behind the others' (one pair of products
+            # serves all), unless steps may take the chosen pairs only: then it keeps matrices and products of its own
+            self.shared_packed = bool(spec.shared_size) and not self._grouped_possible()
+            shared_rows = [tensors["shared.gate"], tensors["shared.up"]] if spec.shared_size else []
+            self.w_gate_up = torch.cat([tensors[f"gate.{e}"] for e in range(n_e)] + [tensors[f"up.{e}"] for e in range(n_e)]
+                                       + (shared_rows if self.shared_packed else []), dim=0).contiguous()
+            self.w_down = torch.cat([tensors[f"down.{e}"] for e in range(n_e)]
+                                    + ([tensors["shared.down"]] if self.shared_packed else []), dim=1).contiguous()
+            if spec.shared_size and not self.shared_packed:
+                self.w_shared_gate_up = torch.cat(shared_rows, dim=0).contiguous()
+                self.w_shared_down = tensors["shared.down"]
+
+    def _grouped_possible(self) -> bool:
+        spec = self.spec
+        return (spec.grouped and self.rt.ops.use_fast_kernels and self.rt.dtype == torch.bfloat16
+                and spec.expert_size * spec.hidden_size >= spec.grouped_min_weight)
 
     def wants_grouped(self, n: int) -> bool:
         """Whether a step of n rows computes the chosen pairs only (where the kernels take the sizes)."""
@@ -114,36 +150,66 @@ class RoutedExperts(FeedForward):
         return (spec.grouped and n * spec.top < spec.grouped_max_rows * spec.num_experts
                 and spec.expert_size * spec.hidden_size >= spec.grouped_min_weight)
 
+    def _grouped(self, x: torch.Tensor, ctx, dense, ids, weights, y) -> bool:
+        """The chosen (token, expert) pairs only: sorted by expert on the device, tiles of 64 rows through MFMA.
+        False: the sizes are not served."""
+        spec, rt, ops, ws = self.spec, self.rt, self.rt.ops, self.rt.workspace
+        n, n_e, F = x.shape[0], spec.num_experts, spec.expert_size
+        need = int(ops.lib.dll.mv_moe_grouped_ints(n, spec.top, n_e)) if ops.lib.has("mv_moe_grouped") else 0
+        return bool(need) and ops.moe_grouped(
+            x, self.w_gate_up, self.w_down, n_e, spec.identity_experts, F, ids, weights, dense,
+            ws.get("moe.ints", (need,), torch.int32), ws.get("moe.pair_act", (n * spec.top, F), rt.dtype),
+            ws.get("moe.pair_out", (n * spec.top, spec.hidden_size), torch.float32), y,
+            limit=spec.limit if spec.activation == "clamped" else 0.0, slope=spec.gate_slope)
+
+    def _add_shared(self, x: torch.Tensor, y: torch.Tensor) -> None:
+        """y += the shared expert's output, as two products of its own."""
+        spec, rt, ops, ws = self.spec, self.rt, self.rt.ops, self.rt.workspace
+        n, FS = x.shape[0], spec.shared_size
+        if spec.activation != "swiglu":
+            raise NotImplementedError("a shared expert with matrices of its own is a gated SiLU pair")
+        act = ws.get("moe.shared_act", (n, FS), rt.dtype)
+        if not ops.gemm_swiglu(x, self.w_shared_gate_up, act):
+            gu = ws.get("moe.shared_gate_up", (n, 2 * FS), rt.dtype)
+            ops.gemm(x, self.w_shared_gate_up, gu)
+            ops.swiglu(gu, act)
+        ys = ws.get("moe.shared_out", (n, spec.hidden_size), rt.dtype)
+        ops.gemm(act, self.w_shared_down, ys)
+        ops.add_rows(y, ys)
+
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         spec, rt, ops, ws = self.spec, self.rt, self.rt.ops, self.rt.workspace
         if not isinstance(x, torch.Tensor):
             x = x.materialize()
         n, E, n_e, F = x.shape[0], spec.router_outputs, spec.num_experts, spec.expert_size
-        logits = ws.get("moe.logits", (n, E), torch.float32)
-        ops.gemm(x, self.w_router, logits)
+        FS = spec.shared_size if n_e and self.shared_packed else 0
+        apart = bool(spec.shared_size) and not FS
         dense = ws.get("moe.dense", (n, E), torch.float32)
         ids = ws.get("moe.ids", (n, spec.top), torch.int32)
         weights = ws.get("moe.weights", (n, spec.top), torch.float32)
-        ops.moe_route(logits, self.correction, spec.groups, spec.keep_groups, spec.top, spec.weight_sum_eps, dense, ids, weights,
-                      scoring=spec.scoring, group_worth=spec.group_worth, normalize=spec.normalize)
+        if spec.router == "table":
+            ops.moe_table_route(ctx.token_ids, self.table, n_e, dense, ids, weights)
+        else:
+            logits = ws.get("moe.logits", (n, E), torch.float32)
+            ops.gemm(x, self.w_router, logits)
+            ops.moe_route(logits, self.correction, spec.groups, spec.keep_groups, spec.top, spec.weight_sum_eps, dense, ids, weights,
+                          scoring=spec.scoring, group_worth=spec.group_worth, normalize=spec.normalize)
         y = ws.get("ffn.out", (n, spec.hidden_size), rt.dtype)
-        if n_e and ops.use_fast_kernels and self.wants_grouped(n):
-            # the chosen (token, expert) pairs only: sorted by expert on the device, tiles of 64 rows through MFMA
-            need = int(ops.lib.dll.mv_moe_grouped_ints(n, spec.top, n_e)) if ops.lib.has("mv_moe_grouped") else 0
-            if need and ops.moe_grouped(x, self.w_gate_up, self.w_down, n_e, spec.identity_experts, F, ids, weights, dense,
-                                        ws.get("moe.ints", (need,), torch.int32), ws.get("moe.pair_act", (n * spec.top, F), rt.dtype),
-                                        ws.get("moe.pair_out", (n * spec.top, spec.hidden_size), torch.float32), y,
-                                        limit=spec.limit if spec.activation == "clamped" else 0.0, slope=spec.gate_slope):
-                return y
+        if n_e and ops.use_fast_kernels and self.wants_grouped(n) and self._grouped(x, ctx, dense, ids, weights, y):
+            if apart:
+                self._add_shared(x, y)
+            return y
         if n_e:
-            gu = ws.get("moe.gate_up", (n, 2 * n_e * F), rt.dtype)
+            gu = ws.get("moe.gate_up", (n, 2 * n_e * F + 2 * FS), rt.dtype)
             ops.gemm(x, self.w_gate_up, gu)
-            act = ws.get("moe.act", (n, n_e * F), rt.dtype)
+            act = ws.get("moe.act", (n, n_e * F + FS), rt.dtype)
             if spec.activation == "clamped":
-                ops.moe_swiglu_scale(gu, dense, n_e, F, act, limit=spec.limit, slope=spec.gate_slope)
+                ops.moe_swiglu_scale(gu, dense, n_e, F, act, limit=spec.limit, slope=spec.gate_slope, shared=FS)
             else:
-                ops.moe_swiglu_scale(gu, dense, n_e, F, act)
+                ops.moe_swiglu_scale(gu, dense, n_e, F, act, shared=FS)
             ops.gemm(act, self.w_down, y)
+            if apart:
+                self._add_shared(x, y)
         if spec.identity_experts or not n_e:
             ops.moe_identity_add(y, x, dense, n_e, spec.identity_experts, overwrite=not n_e)
         return y

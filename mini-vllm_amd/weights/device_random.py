@@ -9,7 +9,7 @@ from typing import Dict, List, Tuple
 import torch
 
 from ..parts.base import TensorDecl
-from .random_init import DEFAULT_STD, _tensor_seed
+from .random_init import DEFAULT_STD, _tensor_seed, random_integers
 from .source import TensorSource
 
 
@@ -37,8 +37,10 @@ class DeviceRandomSource(TensorSource):
         gen = torch.Generator(device=self.device)
         gen.manual_seed(_tensor_seed(self.seed, name))
         if decl.integer:
-            return torch.randint(0, 2 ** 15, decl.shape, generator=gen, dtype=torch.int32, device=self.device)
+            return random_integers(decl, gen, self.device)
         t = torch.randn(decl.shape, generator=gen, dtype=torch.float32, device=self.device) * self.std
         if decl.init == "ones_normal":
             t += 1.0
+        elif decl.init == "identity_normal":
+            t += torch.eye(decl.shape[0], decl.shape[1], dtype=torch.float32, device=self.device)
         return t.to(self.dtype)

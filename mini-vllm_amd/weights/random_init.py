@@ -25,15 +25,30 @@ def _tensor_seed(seed: int, name: str) -> int:
     return int.from_bytes(digest[:8], "little") & 0x7FFFFFFFFFFFFFFF
 
 
+def random_integers(decl: TensorDecl, gen: torch.Generator, device) -> torch.Tensor:
+    """int32 of the declared shape: anything below 2^15, or, for the law "distinct_below:N" on a matrix, rows of
+    distinct numbers below N (a table that names each row's experts)."""
+    if decl.init.startswith("distinct_below:"):
+        below = int(decl.init.split(":")[1])
+        rows, count = decl.shape
+        if count > below:
+            raise ValueError(f"{count} distinct numbers below {below} do not exist")
+        order = torch.rand((rows, below), generator=gen, dtype=torch.float32, device=device).argsort(dim=1)
+        return order[:, :count].to(torch.int32).contiguous()
+    return torch.randint(0, 2 ** 15, decl.shape, generator=gen, dtype=torch.int32, device=device)
+
+
 def random_tensor(name: str, decl: TensorDecl, seed: int, dtype: torch.dtype, std: float = DEFAULT_STD,
                   device: str = "cpu") -> torch.Tensor:
     gen = torch.Generator(device=device)
     gen.manual_seed(_tensor_seed(seed, name))
     if decl.integer:
-        return torch.randint(0, 2 ** 15, decl.shape, generator=gen, dtype=torch.int32, device=device)
+        return random_integers(decl, gen, device)
     t = torch.randn(decl.shape, generator=gen, dtype=torch.float32, device=device) * std
     if decl.init == "ones_normal":
         t += 1.0
+    elif decl.init == "identity_normal":          # a square matrix near the identity
+        t += torch.eye(decl.shape[0], decl.shape[1], dtype=torch.float32, device=device)
     elif decl.init not in ("normal", "zeros_normal"):
         raise ValueError(f"unknown init law {decl.init!r} for {name}")
     return t.to(dtype)
