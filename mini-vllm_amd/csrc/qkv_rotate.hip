@@ -83,6 +83,98 @@ qkv_rotate_norm_store_kernel(T* __restrict__ qkv, long row_stride, int q_off, in
     for (int d = lane; d < D; d += MV_WAVE) dst[d] = from_f<T>(x[d] * inv * (has_weight ? w.at(d) : 1.f));
 }
 
+// The same for heads of 64, 128 or 256 channels that are rotated over all of them in half-split pairs (or not at all),
+// with values as large as keys and everything 16-byte aligned: a head is spread over L = D / 8 neighbouring lanes,
+// eight channels each, read and written 16 bytes at a time; rotation partners and the sum of squares travel by lane
+// shuffles. `store_v` 0: the blended values are written back into the rows and a tiled launch takes them to their
+// pages (steps of many tokens, where a store per token and head would scatter two bytes at a time); 1: they go to
+// their page from here.
+template <typename T, int L>
+__global__ void __launch_bounds__(256)
+qkv_rotate_norm_store_vec_kernel(T* __restrict__ qkv, long row_stride, int q_off, int k_off, int v_off,
+                                 const int* __restrict__ positions, const int* __restrict__ token_seq,
+                                 const int* __restrict__ block_table, int bt_width, int page_size, T* __restrict__ k_pages,
+                                 T* __restrict__ v_pages, int n, int H, int Hkv, WeightPtr qw, WeightPtr kw, int has_weight,
+                                 int unit_norm, float eps, const float* __restrict__ table, const T* __restrict__ mix_rows,
+                                 long mix_stride, WeightPtr mix_weight, int store_v) {
+    constexpr int D = 8 * L;
+    const int heads = H + 2 * Hkv;
+    const long gid = (long)blockIdx.x * 256 + threadIdx.x;
+    const long hidx = gid / L;
+    const int j = (int)(gid % L);
+    const int tok = (int)(hidx / heads), head = (int)(hidx % heads);
+    const int seq = tok < n ? token_seq[tok] : -1;
+    const bool active = tok < n && seq >= 0;          // (inactive lanes still take part in the shuffles)
+    const int pos = active ? positions[tok] : 0;
+    const int kind = head >= H + Hkv ? 2 : (head >= H ? 1 : 0);
+    const int hh = kind == 2 ? head - H - Hkv : (kind == 1 ? head - H : head);
+    T* src = qkv + (size_t)(active ? tok : 0) * row_stride + (kind == 0 ? q_off : (kind == 1 ? k_off : v_off)) + (size_t)hh * D + 8 * j;
+    float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (active) Vec8<T>::load(src, x);
+    if (kind == 2) {
+        if (!active) return;
+        if (mix_rows != nullptr) {
+            const float m = mix_weight.at(0);
+            float o[8];
+            Vec8<T>::load(mix_rows + (size_t)tok * mix_stride + (size_t)hh * D + 8 * j, o);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = (1.f - m) * x[e] + m * o[e];
+            if (!store_v) Vec8<T>::store(src, x);
+        }
+        if (!store_v) return;
+        const int page = block_table[(size_t)seq * bt_width + pos / page_size];
+        if (page < 0) return;
+        T* dst = v_pages + (((size_t)page * Hkv + hh) * D + 8 * j) * page_size + pos % page_size;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dst[(size_t)e * page_size] = from_f<T>(x[e]);
+        return;
+    }
+    if (table != nullptr) {
+        const float* cs = table + (size_t)pos * D + 8 * (j % (L / 2));
+        float c[8], sn[8];
+        Vec8<float>::load(cs, c);
+        Vec8<float>::load(cs + D / 2, sn);
+        const bool low = j < L / 2;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float other = __shfl_xor(x[e], L / 2, MV_WAVE);
+            x[e] = low ? x[e] * c[e] - other * sn[e] : x[e] * c[e] + other * sn[e];
+        }
+    }
+    float inv = 1.f;
+    if (unit_norm) {
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss = fmaf(x[e], x[e], ss);
+#pragma unroll
+        for (int o = L / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, MV_WAVE);
+        inv = 1.f / sqrtf(ss / (float)D + eps);
+    }
+    if (!active) return;
+    if (has_weight) {
+        float w[8];
+        (kind == 0 ? qw : kw).at8(8 * j, w);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] *= w[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] *= inv;
+    if (kind == 0) {
+        Vec8<T>::store(src, x);
+        return;
+    }
+    const int page = block_table[(size_t)seq * bt_width + pos / page_size];
+    if (page < 0) return;
+    Vec8<T>::store(k_pages + (((size_t)page * Hkv + hh) * page_size + pos % page_size) * D + 8 * j, x);
+}
+
+extern "C" int mv_store_v_pages(const void* qkv, long row_stride, int v_off, const int* positions, const int* token_seq,
+                                const int* block_table, int bt_width, int page_size, void* v_pages, int n, int Hkv, int D,
+                                int dtype, hipStream_t stream);
+
+// steps of at least this many tokens write their values tile by tile in a launch of their own
+#define QR_TILED_V_TOKENS 64
+
 extern "C" int mv_qkv_rotate_norm_store(void* qkv, long row_stride, int q_off, int k_off, int v_off, const int* positions,
                                         const int* token_seq, const int* block_table, int bt_width, int page_size,
                                         void* k_pages, void* v_pages, int n, int H, int Hkv, int D, int Dv,
@@ -103,6 +195,30 @@ extern "C" int mv_qkv_rotate_norm_store(void* qkv, long row_stride, int q_off, i
     MV_REQUIRE(H + 2 * Hkv <= 4 * 65535, "qkv_rotate_norm_store: too many heads");
     if (n == 0) return 0;
     WeightPtr qw{q_weight, weight_dtype}, kw{k_weight, weight_dtype}, mw{mix_weight, mix_weight_dtype};
+    const size_t esz = mv_dtype_size(dtype);
+    const bool aligned = ((uintptr_t)qkv % 16) == 0 && (row_stride * esz) % 16 == 0 && (q_off * esz) % 16 == 0 &&
+                         (k_off * esz) % 16 == 0 && (v_off * esz) % 16 == 0 && ((uintptr_t)k_pages % 16) == 0 &&
+                         ((uintptr_t)q_weight % 16) == 0 && ((uintptr_t)k_weight % 16) == 0 && ((uintptr_t)table % 16) == 0 &&
+                         ((uintptr_t)mix_rows % 16) == 0 && (mix_stride * esz) % 16 == 0;
+    if (aligned && D == Dv && (D == 64 || D == 128 || D == 256) && (table == nullptr || (rot_dim == D && !interleaved)) &&
+        (long)n * (H + 2 * Hkv) * (D / 8) < (1L << 31)) {
+        const int store_v = n < QR_TILED_V_TOKENS;
+        const long lanes = (long)n * (H + 2 * Hkv) * (D / 8);
+        const dim3 vgrid((unsigned)((lanes + 255) / 256));
+#define QR_VEC(LL)                                                                                                          \
+    MV_DISPATCH_T(dtype, "qkv_rotate_norm_store",                                                                           \
+                  hipLaunchKernelGGL((qkv_rotate_norm_store_vec_kernel<T, LL>), vgrid, dim3(256), 0, stream, (T*)qkv,       \
+                                     row_stride, q_off, k_off, v_off, positions, token_seq, block_table, bt_width, page_size, \
+                                     (T*)k_pages, (T*)v_pages, n, H, Hkv, qw, kw, q_weight != nullptr, unit_norm, eps, table, \
+                                     (const T*)mix_rows, mix_stride, mw, store_v))
+        if (D == 64) { QR_VEC(8); } else if (D == 128) { QR_VEC(16); } else { QR_VEC(32); }
+#undef QR_VEC
+        if (int rc = mv_check_launch("qkv_rotate_norm_store")) return rc;
+        if (!store_v)
+            return mv_store_v_pages(qkv, row_stride, v_off, positions, token_seq, block_table, bt_width, page_size, v_pages, n,
+                                    Hkv, Dv, dtype, stream);
+        return 0;
+    }
     dim3 grid(n, (H + 2 * Hkv + 3) / 4);
     MV_DISPATCH_T(dtype, "qkv_rotate_norm_store",
                   hipLaunchKernelGGL(qkv_rotate_norm_store_kernel<T>, grid, dim3(256), 0, stream, (T*)qkv, row_stride, q_off,

@@ -260,3 +260,8 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int], start: int
     if rnd:
         hn = rnd(hn)
     return hn @ w["embed"].T, new_past
+
+
+def round_to_bfloat16(t: torch.Tensor) -> torch.Tensor:
+    """What an engine that stores activations in bfloat16 keeps of ``t`` (round to nearest even)."""
+    return t.to(torch.bfloat16).to(t.dtype)
