@@ -42,6 +42,10 @@ attention over a window of ``--window`` positions beside the first ``--keep-firs
 feed-forward dense and the others mixtures of ``--experts`` experts of which a token uses ``--top``); with
 ``--dense-every 1`` every feed-forward is dense, which is the model to read beside Qwen3 of the same shape.
 
+``--design furanex`` does the same for a Furanex model of the named shape's sizes (``furanex_shape``: ``--streams``
+residual streams; grouped attention whose values are shared along the layers alternating with attention over a latent;
+every feed-forward a mixture of ``--experts`` experts named by a table, ``--top`` a token, beside a shared expert).
+
 Weights are seeded random tensors of the named shape and prompts are seeded uniform token ids
 (there is no network for checkpoints or datasets). The reference publishes no number for this
 metric, so ``vs_baseline`` is null.
@@ -93,6 +97,10 @@ def build_llm(args, shape, layers, max_seqs=None, token_budget=None, num_pages=N
         from minivllm_amd.config.shapes import zedudra_shape
         raw = dict(zedudra_shape(args.shape, layers, window=args.window, keep_first=args.keep_first, experts=args.experts,
                                  top=args.top, dense_every=args.dense_every), torch_dtype=args.dtype)
+    elif getattr(args, "design", "qwen3") == "furanex":
+        from minivllm_amd.config.shapes import furanex_shape
+        raw = dict(furanex_shape(args.shape, layers, streams=args.streams, experts=args.experts, top=args.top,
+                                 latent_every=args.latent_every), torch_dtype=args.dtype)
     else:
         raw = dict(shape, architectures=["Qwen3ForCausalLM"], num_hidden_layers=layers,
                    max_position_embeddings=40960, torch_dtype=args.dtype)
@@ -449,6 +457,77 @@ def bench_dutilix(args, llm, cfg, layers, layers_full, item) -> int:
     return 0
 
 
+def furanex_numbers(llm, cfg, item):
+    """From the loaded model: elements of all tensors; of the matrices every token multiplies with (the shared experts
+    among them); of all routed experts and of those a token uses; cache bytes a token takes in each layer."""
+    from minivllm_amd.models.causal_lm import expected_tensors
+    ex = llm.executor
+    decls = expected_tensors(ex.arch, cfg, ex.plan)
+    params = sum(_numel(d.shape) for d in decls.values())
+    routed = lambda n: ".mlp.e" in n
+    expert = sum(_numel(d.shape) for n, d in decls.items() if routed(n))
+    matrices = sum(_numel(d.shape) for n, d in decls.items() if len(d.shape) == 2 and n != "embed" and not routed(n)
+                   and not n.endswith((".table", ".mix")))
+    routers = [(l.mlp.experts, l.mlp.top) for l in cfg.layers if l.mlp is not None]
+    per_layer_expert = expert // max(1, len(routers))
+    active = sum(per_layer_expert * min(t, e) // max(e, 1) for e, t in routers)
+    cache = [2 * l.mixer.kv_heads * (l.mixer.dim + l.mixer.vdim) // 2 if l.mixer.kind == "attention"
+             else 2 * l.mixer.kv_rank + l.mixer.rot_dim for l in cfg.layers]           # elements a token, a layer
+    # multiply-adds of a (query, key) pair: grouped attention q.k and p.v; over a latent (R + Dr) + R a head
+    pair = [l.mixer.heads * (l.mixer.dim + l.mixer.vdim) if l.mixer.kind == "attention"
+            else l.mixer.heads * (2 * l.mixer.kv_rank + l.mixer.rot_dim) for l in cfg.layers]
+    return dict(params=params, matrices=matrices, expert=expert, active=active, routers=routers,
+                per_layer_expert=per_layer_expert, cache=cache, pair=pair)
+
+
+def bench_furanex(args, llm, cfg, layers, layers_full, item) -> int:
+    """The default measurements for a Furanex model of the named shape; the same fields in the line."""
+    nums = furanex_numbers(llm, cfg, item)
+    prefill = None
+    if args.only in ("all", "prefill"):
+        prefill_s = measure_prefill(llm, cfg.vocab_size, args.prefill_tokens, repeats=3, seed=args.seed)
+        T = args.prefill_tokens
+        flops = 2 * T * (nums["matrices"] + nums["active"]) + 2 * cfg.vocab_size * cfg.hidden_size
+        flops += sum(2 * p * T * (T + 1) // 2 for p in nums["pair"])
+        prefill = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+                   "frac": round(flops / prefill_s / PEAK_FLOPS[args.dtype], 4)}
+    tok_s = ms_step = roofline = None
+    ran = regions = 0
+    if args.only in ("all", "decode"):
+        tok_s, ms_step, mean_ctx, ran, regions = measure_decode(llm, cfg.vocab_size, args.batch, args.prompt_len,
+                                                                args.steps, args.warmup, args.seed)
+        # every weight that some request of the step uses once (of a layer's E experts about E (1 - (1 - top/E)^batch)),
+        # each request's cache once, the residual streams read and written between the sublayers
+        touched = sum(nums["per_layer_expert"] * (1.0 - (1.0 - min(t, e) / e) ** args.batch) for e, t in nums["routers"])
+        lanes = 2 * len(cfg.layers) * 2 * max(cfg.streams, 1) * cfg.hidden_size * 4
+        step_bytes = (nums["params"] - nums["expert"] + touched) * item + args.batch * (sum(nums["cache"]) * item * mean_ctx + lanes)
+        achieved = step_bytes / (ms_step * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(achieved / PEAK_HBM_GBS, 4)}
+    points = {}
+    if not args.no_points and args.only == "all":
+        for b, key in ((1, "decode_b1"), (64, "decode_b64")):
+            n = min(args.steps, 128)
+            points[key] = round(measure_decode(llm, cfg.vocab_size, b, args.prompt_len, n, min(args.warmup, 8),
+                                               args.seed + b)[0], 1)
+    config = {"model": f"furanex-{args.shape}-shape-random", "layers": layers, "layers_full": layers_full,
+              "hidden": cfg.hidden_size, "vocab": cfg.vocab_size, "streams": cfg.streams,
+              "latent_layers": sum(1 for l in cfg.layers if l.mixer.kind == "latent_attention"),
+              "experts": args.experts, "top": args.top, "weights": nums["params"],
+              "weights_a_token_uses": nums["params"] - nums["expert"] + nums["active"], "global_batch": args.batch,
+              "seq_len": args.context, "prompt_len": args.prompt_len, "block_size": args.block_size, "graph": not args.no_graph,
+              "scheduler_steps": args.scheduler_steps, "launch_ahead": bool(llm.config.launch_ahead),
+              "parallelism": "single-gpu"}
+    print(json.dumps({"metric": "decode tok/s (batch %d, %d-token prompts)" % (args.batch, args.prompt_len),
+                      "value": round(tok_s, 1) if tok_s is not None else None, "unit": "tokens/s", "n_gpus": 1,
+                      "steps": ran if ran else args.steps, "warmup": args.warmup,
+                      "ms_per_step": round(ms_step, 4) if ms_step is not None else None, "higher_is_better": True,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                      "data": "synthetic", "config": config, "timed_regions": regions, "prefill": prefill,
+                      "roofline": roofline, "points": points}))
+    return 0
+
+
 def zedudra_numbers(llm, cfg, item):
     """From the loaded model: elements of all tensors; of the matrices every token multiplies with; of all expert
     matrices and of those a token uses; bytes of convolution state a request reads and writes a step; cache bytes a
@@ -535,7 +614,11 @@ def main() -> int:
     ap.add_argument("--dense-every", type=int, default=2,
                     help="--design zedudra: every n-th feed-forward is dense, the others are routed (1: all dense; a number "
                          "above the layer count: only the first)")
-    ap.add_argument("--design", choices=["qwen3", "bolapel", "dutilix", "zedudra"], default="qwen3",
+    ap.add_argument("--streams", type=int, default=4, help="--design furanex: residual streams")
+    ap.add_argument("--latent-every", type=int, default=2,
+                    help="--design furanex: every n-th layer attends over a latent, the others are grouped attention (a number "
+                         "above the layer count: grouped attention everywhere)")
+    ap.add_argument("--design", choices=["qwen3", "bolapel", "dutilix", "zedudra", "furanex"], default="qwen3",
                     help="'bolapel': the same widths, head counts, vocabulary and number of layers as the named Qwen3 "
                          "shape, as a Bolapel model (three delta-rule layers to one attention layer in chunks of --chunk "
                          "tokens); decode and prefill are measured the same way and the line names the design")
@@ -640,6 +723,8 @@ def main() -> int:
         return bench_dutilix(args, llm, cfg, layers, layers_full, item)
     if args.design == "zedudra":
         return bench_zedudra(args, llm, cfg, layers, layers_full, item)
+    if args.design == "furanex":
+        return bench_furanex(args, llm, cfg, layers, layers_full, item)
     nums = model_numbers(shape, layers)
 
     prefill = None

@@ -26,6 +26,7 @@ _LIBRARY = r"^((Custom_)?Cijk_|void hipblaslt|hipblaslt|.*rocblaslt)"
 # most kernels one call launches)
 KERNELS_OF: Dict[str, Tuple[str, Optional[str], int]] = {
     "mv_embedding": (r"\bembedding(_gather)?_kernel", None, 1),
+    "mv_gather_rows": (r"\bembedding_kernel", None, 1),
     "mv_add_rmsnorm": (r"\badd_rmsnorm(_vec)?_kernel", None, 1),
     "mv_add_rmsnorm_split": (r"\badd_rmsnorm(_vec)?_kernel", None, 1),
     "mv_rmsnorm": (r"\brmsnorm_kernel", None, 1),
@@ -75,6 +76,10 @@ KERNELS_OF: Dict[str, Tuple[str, Optional[str], int]] = {
     "mv_group_norm_add_norm": (r"\bgroup_norm_add_norm(_vec)?_kernel", None, 1),
     "mv_xielu": (r"\bxielu(_vec)?_kernel", None, 1),
     "mv_moe_grouped": (r"\bmoe_sort_kernel", r"\bmoe_(expert_product|combine)_kernel", 4),
+    "mv_hyper_step": (r"\bhyper_step(_vec)?_kernel", None, 1),
+    "mv_qkv_rotate_norm_store": (r"\bqkv_rotate_norm_store(_vec)?_kernel", r"\bstore_v_pages_kernel", 2),
+    "mv_moe_table_route": (r"\bmoe_table_route_kernel", None, 1),
+    "mv_add_rows": (r"\badd_rows_kernel", None, 1),
 }
 _OURS = re.compile("|".join(f"(?:{p})" for spec in KERNELS_OF.values() for p in spec[:2] if p))
 

@@ -277,7 +277,7 @@ class Ops:
         """out[n] = table[index[n]] for a float32 table (rows outside it give zeros)."""
         n = out.shape[0]
         self._check_gather(index, table, out, n)
-        self._note("mv_embedding", n * (8 * out.shape[1] + 4))
+        self._note("mv_gather_rows", n * (8 * out.shape[1] + 4))      # (a name of its own: "mv_embedding" starts a model step)
         self.lib.call("mv_embedding", index.data_ptr(), table.data_ptr(), DTYPE_F32, out.data_ptr(), n, table.shape[1],
                       table.shape[0], 1.0, self._stream())
 
