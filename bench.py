@@ -482,6 +482,7 @@ def furanex_numbers(llm, cfg, item):
 
 def bench_furanex(args, llm, cfg, layers, layers_full, item) -> int:
     """The default measurements for a Furanex model of the named shape; the same fields in the line."""
+    cfg = llm.executor.model_config            # (with every size stated)
     nums = furanex_numbers(llm, cfg, item)
     prefill = None
     if args.only in ("all", "prefill"):

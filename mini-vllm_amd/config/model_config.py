@@ -945,6 +945,15 @@ class ZedudraConfig(ModelConfig):
 # ---------------------------------------------------------------------------------------
 # Furanex
 # ---------------------------------------------------------------------------------------
+UNSTATED = -1          # a size that config.json leaves to the shapes of the stored tensors (``furanex_complete`` fills it in)
+
+
+def _size(d: Dict[str, Any], key: str, where: str) -> int:
+    """An integer size of config.json, or UNSTATED when the key is absent."""
+    v = d.get(key)
+    return UNSTATED if v is None else _typed(v, key, int, where)
+
+
 @dataclass(frozen=True)
 class FuranexRotation:
     """Rotation by position over the first ``dims`` channels; ``stretch`` = (factor, original, fast, slow) slows the
@@ -964,18 +973,19 @@ class FuranexRotation:
 class FuranexMixer:
     """``kind`` "attention": ``heads`` query heads on ``kv_heads`` key/value heads, keys of ``dim`` and values of ``vdim``
     channels, ``v_mix``: the values are shared along the layers. ``kind`` "latent_attention": ``heads`` heads with ``dim``
-    unrotated and ``rot_dim`` rotated query/key channels, values of ``vdim``, latents of ``q_rank`` and ``kv_rank``."""
+    unrotated and ``rot_dim`` rotated query/key channels, values of ``vdim``, latents of ``q_rank`` and ``kv_rank``.
+    A size may be UNSTATED, and ``scale`` None, until the configuration has been completed."""
     kind: str
     heads: int
     dim: int
     vdim: int
-    scale: float
+    scale: Optional[float]
     rot: Optional[FuranexRotation] = None
-    kv_heads: int = 0
+    kv_heads: int = UNSTATED
     v_mix: bool = False
-    rot_dim: int = 0
-    q_rank: int = 0
-    kv_rank: int = 0
+    rot_dim: int = UNSTATED
+    q_rank: int = UNSTATED
+    kv_rank: int = UNSTATED
 
     def to_dict(self) -> Dict[str, Any]:
         d: Dict[str, Any] = {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale}
@@ -985,7 +995,7 @@ class FuranexMixer:
             d.update(kv_heads=self.kv_heads, v_mix=self.v_mix)
         else:
             d.update(rot_dim=self.rot_dim, q_rank=self.q_rank, kv_rank=self.kv_rank)
-        return d
+        return {k: v for k, v in d.items() if v is not None and v != UNSTATED}
 
 
 @dataclass(frozen=True)
@@ -995,12 +1005,18 @@ class FuranexFeedForward:
     ff: int
     experts: int
     top: int
-    shared_ff: int = 0
+    shared_ff: int = UNSTATED
 
     def to_dict(self) -> Dict[str, Any]:
-        d: Dict[str, Any] = {"kind": "moe", "expert": {"ff": self.ff}, "router": {"experts": self.experts, "top": self.top}}
-        if self.shared_ff:
-            d["shared"] = {"ff": self.shared_ff}
+        d: Dict[str, Any] = {"kind": "moe", "expert": {}, "router": {}}
+        if self.ff != UNSTATED:
+            d["expert"]["ff"] = self.ff
+        if self.experts != UNSTATED:
+            d["router"]["experts"] = self.experts
+        if self.top != UNSTATED:
+            d["router"]["top"] = self.top
+        if self.shared_ff != UNSTATED:
+            d["shared"] = {"ff": self.shared_ff} if self.shared_ff else None
         return d
 
 
@@ -1016,13 +1032,15 @@ class FuranexConfig(ModelConfig):
     softmax attention (rotation first, then a unit norm of q and k; values blended with the first such layer's) or
     attention over a cached latent with a gate per head; feed-forwards whose experts a table names by token id, beside a
     shared expert. The embedding is multiplied by ``embedding.scale``; the output head is the embedding's table.
-    Keys: ``vocab``, ``width``, ``streams``, ``layers``, ``norm.eps``, ``embedding.scale``."""
+    Keys: ``vocab``, ``width``, ``streams``, ``layers``, ``norm.eps``, ``embedding.scale``. Sizes that config.json leaves
+    out are UNSTATED until ``completed`` has filled them in, from the stored tensors' shapes (``models/furanex.py``) or
+    with their defaults (``kv_heads`` = heads, ``vdim`` = dim, ``rot_dim`` = rot.dims, no shared expert, one residual)."""
 
     architecture: ClassVar[str] = "Furanex"
 
-    vocab_size: int = 0
-    hidden_size: int = 0
-    streams: int = 0                       # 0: one plain residual
+    vocab_size: int = UNSTATED
+    hidden_size: int = UNSTATED
+    streams: int = UNSTATED                # 0: one plain residual
     layers: Tuple[FuranexLayer, ...] = ()
     norm_eps: float = 1e-6
     embedding_scale: float = 1.0
@@ -1053,43 +1071,36 @@ class FuranexConfig(ModelConfig):
             if not isinstance(entry, dict):
                 raise ConfigError(f"{lw} must be an object")
             kind = entry.get("type")
+            if kind not in ("attention", "latent_attention"):
+                raise ConfigError(f"{lw}: layer type {kind!r} is not supported (attention, latent_attention)")
             m = _section(entry, "mixer", lw)
             mw = lw + ".mixer"
-            heads, dim = _require(m, "heads", int, mw), _require(m, "dim", int, mw)
-            vdim, scale = m.get("vdim"), m.get("scale")
-            rot = cls._rotation(m, mw)
-            common = dict(kind=kind, heads=heads, dim=dim, vdim=dim if vdim is None else _typed(vdim, "vdim", int, mw), rot=rot)
-            if kind == "attention":
-                kv_heads, v_mix = m.get("kv_heads"), m.get("v_mix")
-                mixer = FuranexMixer(scale=dim ** -0.5 if scale is None else _typed(scale, "scale", float, mw),
-                                     kv_heads=heads if kv_heads is None else _typed(kv_heads, "kv_heads", int, mw),
-                                     v_mix=False if v_mix is None else _typed(v_mix, "v_mix", bool, mw), **common)
-            elif kind == "latent_attention":
-                rot_dim = m.get("rot_dim")
-                rot_dim = (rot.dims if rot is not None else 0) if rot_dim is None else _typed(rot_dim, "rot_dim", int, mw)
-                mixer = FuranexMixer(scale=(dim + rot_dim) ** -0.5 if scale is None else _typed(scale, "scale", float, mw),
-                                     rot_dim=rot_dim, q_rank=_require(m, "q_rank", int, mw),
-                                     kv_rank=_require(m, "kv_rank", int, mw), **common)
-            else:
-                raise ConfigError(f"{lw}: layer type {kind!r} is not supported (attention, latent_attention)")
+            scale, v_mix = m.get("scale"), m.get("v_mix")
+            if kind == "latent_attention" and v_mix:
+                raise ConfigError(f"{mw}: a latent layer caches no values that could be shared along the layers")
+            mixer = FuranexMixer(kind=kind, heads=_size(m, "heads", mw), dim=_size(m, "dim", mw), vdim=_size(m, "vdim", mw),
+                                 scale=None if scale is None else _typed(scale, "scale", float, mw), rot=cls._rotation(m, mw),
+                                 kv_heads=_size(m, "kv_heads", mw), v_mix=False if v_mix is None else _typed(v_mix, "v_mix", bool, mw),
+                                 rot_dim=_size(m, "rot_dim", mw), q_rank=_size(m, "q_rank", mw), kv_rank=_size(m, "kv_rank", mw))
             mlp = _section(entry, "mlp", lw, optional=True)
             ff = None
             if mlp is not None:
                 pw = lw + ".mlp"
                 if mlp.get("kind", "moe") != "moe":
                     raise ConfigError(f"{pw}: kind {mlp.get('kind')!r} is not supported (moe)")
-                expert = _section(mlp, "expert", pw)
-                router = _section(mlp, "router", pw)
-                shared = _section(mlp, "shared", pw, optional=True)
-                ff = FuranexFeedForward(ff=_require(expert, "ff", int, pw + ".expert"),
-                                        experts=_require(router, "experts", int, pw + ".router"),
-                                        top=_require(router, "top", int, pw + ".router"),
-                                        shared_ff=0 if shared is None else _require(shared, "ff", int, pw + ".shared"))
+                expert = _section(mlp, "expert", pw, optional=True) or {}
+                router = _section(mlp, "router", pw, optional=True) or {}
+                if "shared" in mlp:          # stated: a section with its width, or null for none
+                    shared = _section(mlp, "shared", pw, optional=True)
+                    shared_ff = 0 if shared is None else _size(shared, "ff", pw + ".shared")
+                else:
+                    shared_ff = UNSTATED
+                ff = FuranexFeedForward(ff=_size(expert, "ff", pw + ".expert"), experts=_size(router, "experts", pw + ".router"),
+                                        top=_size(router, "top", pw + ".router"), shared_ff=shared_ff)
             layers.append(FuranexLayer(mixer=mixer, mlp=ff))
         norm = _section(d, "norm", where)
         emb = _section(d, "embedding", where, optional=True)
         emb_scale = None if emb is None else emb.get("scale")
-        streams = d.get("streams")
         dtype = d.get("dtype", d.get("torch_dtype", "bfloat16")) or "bfloat16"
         if str(dtype) not in _DTYPE_NAMES:
             raise ConfigError(f"{where}: unknown dtype {dtype!r}")
@@ -1103,9 +1114,7 @@ class FuranexConfig(ModelConfig):
             raise ConfigError(f"{where}: eos_token_id must be an integer or a list of integers, got {eos!r}")
         max_pos = d.get("max_position_embeddings")
         cfg = cls(
-            vocab_size=_require(d, "vocab", int, where),
-            hidden_size=_require(d, "width", int, where),
-            streams=0 if streams is None else _typed(streams, "streams", int, where),
+            vocab_size=_size(d, "vocab", where), hidden_size=_size(d, "width", where), streams=_size(d, "streams", where),
             layers=tuple(layers),
             norm_eps=_require(norm, "eps", float, where + ".norm"),
             embedding_scale=1.0 if emb_scale is None else _typed(emb_scale, "scale", float, where + ".embedding"),
@@ -1123,18 +1132,82 @@ class FuranexConfig(ModelConfig):
                 return i
         return None
 
-    def validate(self, where: str = "config") -> None:
-        if self.vocab_size <= 0 or self.hidden_size <= 0:
+    def completed(self, sizes=None, where: str = "config") -> "FuranexConfig":
+        """The configuration with nothing UNSTATED. ``sizes(name) -> shape or None`` looks a stored tensor's shape up;
+        a size that neither config.json nor a shape states takes its default, or is an error when it has none."""
+        import dataclasses
+        sizes = sizes or (lambda name: None)
+
+        def axis(name: str, k: int) -> Optional[int]:
+            shape = sizes(name)
+            return None if shape is None or len(shape) <= k else int(shape[k])
+
+        def need(value: int, found: Optional[int], what: str, default: Optional[int] = None) -> int:
+            if value != UNSTATED:
+                return value
+            if found is not None:
+                return found
+            if default is not None:
+                return default
+            raise ConfigError(f"{where}: {what} is stated neither in config.json nor by a stored tensor's shape")
+
+        def per(total: Optional[int], count: int) -> Optional[int]:
+            return None if total is None or count in (UNSTATED, 0) or total % count else total // count
+
+        vocab = need(self.vocab_size, axis("embed", 0), "vocab")
+        width = need(self.hidden_size, axis("embed", 1), "width")
+        streams = need(self.streams, axis("l0.hc1.in", 0), "streams", 0)
+        layers = []
+        for i, l in enumerate(self.layers):
+            m, p, lw = l.mixer, f"l{i}.mix.", f"layers[{i}].mixer"
+            if m.kind == "attention":
+                q_rows, k_rows, v_rows = axis(p + "q", 0), axis(p + "k", 0), axis(p + "v", 0)
+                heads = need(m.heads, per(q_rows, m.dim), lw + ".heads")
+                dim = need(m.dim, per(q_rows, heads), lw + ".dim")
+                kv_heads = need(m.kv_heads, per(k_rows, dim), lw + ".kv_heads", heads)
+                vdim = need(m.vdim, per(v_rows, kv_heads), lw + ".vdim", dim)
+                m = dataclasses.replace(m, heads=heads, dim=dim, kv_heads=kv_heads, vdim=vdim, rot_dim=0, q_rank=0, kv_rank=0,
+                                        scale=dim ** -0.5 if m.scale is None else m.scale)
+            else:
+                heads = need(m.heads, axis(p + "g", 0), lw + ".heads")
+                dim = need(m.dim, per(axis(p + "uk", 0), heads), lw + ".dim")
+                vdim = need(m.vdim, per(axis(p + "uv", 0), heads), lw + ".vdim", dim)
+                q_rank = need(m.q_rank, axis(p + "dq.norm", 0), lw + ".q_rank")
+                kv_rank = need(m.kv_rank, axis(p + "dkv.norm", 0), lw + ".kv_rank")
+                rows = axis(p + "dkv", 0)
+                rot_dim = need(m.rot_dim, None if rows is None else rows - kv_rank, lw + ".rot_dim", m.rot.dims if m.rot is not None else 0)
+                m = dataclasses.replace(m, heads=heads, dim=dim, vdim=vdim, q_rank=q_rank, kv_rank=kv_rank, rot_dim=rot_dim, kv_heads=0,
+                                        scale=(dim + rot_dim) ** -0.5 if m.scale is None else m.scale)
+            f = l.mlp
+            if f is not None:
+                y, fw = f"l{i}.mlp.", f"layers[{i}].mlp"
+                counted = 0
+                while sizes(f"{y}e{counted}.gate") is not None:
+                    counted += 1
+                f = FuranexFeedForward(ff=need(f.ff, axis(y + "e0.gate", 0), fw + ".expert.ff"),
+                                       experts=need(f.experts, counted or None, fw + ".router.experts"),
+                                       top=need(f.top, axis(y + "table", 1), fw + ".router.top"),
+                                       shared_ff=need(f.shared_ff, axis(y + "shared.gate", 0), fw + ".shared.ff", 0))
+            layers.append(FuranexLayer(mixer=m, mlp=f))
+        done = dataclasses.replace(self, vocab_size=vocab, hidden_size=width, streams=streams, layers=tuple(layers))
+        done.validate(where, final=True)
+        return done
+
+    def validate(self, where: str = "config", final: bool = False) -> None:
+        """Checks what is stated; with ``final`` nothing may be UNSTATED any more."""
+        known = lambda *values: all(v != UNSTATED and v is not None for v in values)
+        positive = lambda v: v == UNSTATED or v > 0
+        if not positive(self.vocab_size) or not positive(self.hidden_size):
             raise ConfigError(f"{where}: vocab and width must be positive")
         if self.norm_eps <= 0:
             raise ConfigError(f"{where}: norm.eps must be positive, got {self.norm_eps}")
-        if self.streams < 0 or self.streams > 8:
+        if self.streams != UNSTATED and not (0 <= self.streams <= 8):
             raise ConfigError(f"{where}: streams must lie in 1..8, got {self.streams}")
         first = self.first_mixing_layer()
         for i, l in enumerate(self.layers):
             lw = f"{where}: layers[{i}]"
             m = l.mixer
-            if m.heads <= 0 or m.dim <= 0 or m.vdim <= 0 or not m.scale > 0:
+            if not all(positive(v) for v in (m.heads, m.dim, m.vdim)) or (m.scale is not None and not m.scale > 0):
                 raise ConfigError(f"{lw}: heads, dim, vdim and scale must be positive")
             if m.rot is not None:
                 r = m.rot
@@ -1143,21 +1216,28 @@ class FuranexConfig(ModelConfig):
                 if r.stretch is not None and not all(v > 0 for v in r.stretch):
                     raise ConfigError(f"{lw}: rot.scaling needs positive factor, original, fast and slow")
             if m.kind == "attention":
-                if m.kv_heads <= 0 or m.heads % m.kv_heads:
+                if not positive(m.kv_heads) or (known(m.heads, m.kv_heads) and m.heads % m.kv_heads):
                     raise ConfigError(f"{lw}: {m.heads} heads are not a multiple of {m.kv_heads} kv_heads")
-                if m.rot is not None and m.rot.dims > m.dim:
+                if m.rot is not None and known(m.dim) and m.rot.dims > m.dim:
                     raise ConfigError(f"{lw}: rot.dims {m.rot.dims} exceeds dim {m.dim}")
-                if m.v_mix and (self.layers[first].mixer.kv_heads, self.layers[first].mixer.vdim) != (m.kv_heads, m.vdim):
+                f0 = self.layers[first].mixer if first is not None else None
+                if m.v_mix and known(m.kv_heads, m.vdim, f0.kv_heads, f0.vdim) and (f0.kv_heads, f0.vdim) != (m.kv_heads, m.vdim):
                     raise ConfigError(f"{lw}: layers that share their values need the kv_heads and vdim of layer {first}")
             else:
-                if m.q_rank <= 0 or m.kv_rank <= 0 or m.rot_dim < 0 or m.rot_dim % 2:
+                if not positive(m.q_rank) or not positive(m.kv_rank) or (m.rot_dim != UNSTATED and (m.rot_dim < 0 or m.rot_dim % 2)):
                     raise ConfigError(f"{lw}: q_rank and kv_rank must be positive, rot_dim even and >= 0")
-                if (m.rot.dims if m.rot is not None else 0) != m.rot_dim:
+                if known(m.rot_dim) and (m.rot.dims if m.rot is not None else 0) != m.rot_dim:
                     raise ConfigError(f"{lw}: the rotated part has rot_dim {m.rot_dim} channels, so rot.dims must equal it")
             f = l.mlp
             if f is not None:
-                if f.ff <= 0 or f.experts < 1 or not (1 <= f.top <= f.experts) or f.shared_ff < 0:
+                if not positive(f.ff) or not positive(f.experts) or not positive(f.top) or f.shared_ff < UNSTATED \
+                        or (known(f.top, f.experts) and f.top > f.experts):
                     raise ConfigError(f"{lw}: a mixture needs a positive expert width, experts >= 1 and 1 <= top <= experts")
+            if final and not (known(m.heads, m.dim, m.vdim, m.scale, m.kv_heads, m.rot_dim, m.q_rank, m.kv_rank)
+                              and (f is None or known(f.ff, f.experts, f.top, f.shared_ff))):
+                raise ConfigError(f"{lw}: a size is still not stated")
+        if final and not known(self.vocab_size, self.hidden_size, self.streams):
+            raise ConfigError(f"{where}: vocab, width or streams is still not stated")
 
     def to_dict(self) -> Dict[str, Any]:
         layers = [{"type": l.mixer.kind, "mixer": l.mixer.to_dict(), "mlp": None if l.mlp is None else l.mlp.to_dict()}
@@ -1167,12 +1247,11 @@ class FuranexConfig(ModelConfig):
             "layers": layers,
             "norm": {"eps": self.norm_eps},
             "embedding": {"scale": self.embedding_scale},
-            "vocab": self.vocab_size,
-            "width": self.hidden_size,
             "torch_dtype": self.dtype,
         }
-        if self.streams:
-            d["streams"] = self.streams
+        for key, value in (("vocab", self.vocab_size), ("width", self.hidden_size), ("streams", self.streams)):
+            if value != UNSTATED and (key != "streams" or value):
+                d[key] = value
         if self.eos_token_ids:
             d["eos_token_id"] = list(self.eos_token_ids) if len(self.eos_token_ids) > 1 else self.eos_token_ids[0]
         if self.max_position_embeddings != (1 << 24):

@@ -146,41 +146,98 @@ extern "C" int mv_moe_route(const float* logits, long ld, int n, int E, const vo
 }
 
 // gate_up rows: [gate of expert 0 (F) | ... | gate of expert E-1 | up of expert 0 | ... | up of expert E-1 | gate of the
-// shared expert (FS) | its up (FS)]; act rows [E][F] and behind them the shared expert's FS, whose weight is one
+// shared expert (FS) | its up (FS)]; act rows [E][F] and behind them the shared expert's FS, whose weight is one.
+// The weight of (row, expert) comes from `dense`, or, with a table, from the row's token id: 1 / top when
+// table[token][0 .. top) names the expert, else zero (a token id outside the table chooses nothing).
+struct MoeWeights {
+    const float* dense;
+    int ld_dense;
+    const int* tokens;
+    const int* table;
+    int table_rows, top;
+    __device__ __forceinline__ float of(long t, int e) const {
+        if (table == nullptr) return dense[t * ld_dense + e];
+        const int tok = tokens[t];
+        if (tok < 0 || tok >= table_rows) return 0.f;
+        float w = 0.f;
+        for (int k = 0; k < top; ++k)
+            if (table[(size_t)tok * top + k] == e) w += 1.f / (float)top;
+        return w;
+    }
+};
+
+__device__ __forceinline__ float moe_pair(float w, float g, float u, float limit, float slope) {
+    if (limit > 0.f) {
+        const float gc = fminf(g, limit), uc = fminf(fmaxf(u, -limit), limit);
+        return w * (gc / (1.f + expf(-slope * gc))) * (uc + 1.f);
+    }
+    return w * (g / (1.f + expf(-g))) * u;
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256)
-moe_swiglu_scale_kernel(const T* __restrict__ gate_up, long ld, const float* __restrict__ dense, int ld_dense, int E, int F, int FS,
+moe_swiglu_scale_kernel(const T* __restrict__ gate_up, long ld, MoeWeights mw, int E, int F, int FS,
                         T* __restrict__ act, long total, float limit, float slope) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= total) return;
     const long EF = (long)E * F;
     const long t = i / (EF + FS), c = i % (EF + FS);
     const bool shared = c >= EF;
-    const float w = shared ? 1.f : dense[t * ld_dense + c / F];
+    const float w = shared ? 1.f : mw.of(t, (int)(c / F));
     float v = 0.f;
     if (w != 0.f) {
         const long gi = shared ? 2 * EF + (c - EF) : c, ui = shared ? 2 * EF + FS + (c - EF) : EF + c;
-        const float g = to_f(gate_up[t * ld + gi]), u = to_f(gate_up[t * ld + ui]);
-        if (limit > 0.f) {
-            const float gc = fminf(g, limit), uc = fminf(fmaxf(u, -limit), limit);
-            v = w * (gc / (1.f + expf(-slope * gc))) * (uc + 1.f);
-        } else {
-            v = w * (g / (1.f + expf(-g))) * u;
-        }
+        v = moe_pair(w, to_f(gate_up[t * ld + gi]), to_f(gate_up[t * ld + ui]), limit, slope);
     }
     act[t * (EF + FS) + c] = from_f<T>(v);
 }
 
+// The same, eight columns a thread (F and FS multiples of eight, rows 16-byte aligned): a thread's columns belong to
+// one expert, so its weight is looked up once, and the pair of an expert that was not chosen is never loaded.
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_swiglu_scale_vec_kernel(const T* __restrict__ gate_up, long ld, MoeWeights mw, int E, int F, int FS,
+                            T* __restrict__ act, long total8, float limit, float slope) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total8) return;
+    const long EF = (long)E * F;
+    const long row8 = (EF + FS) / 8;
+    const long t = i / row8, c = (i % row8) * 8;
+    const bool shared = c >= EF;
+    const float w = shared ? 1.f : mw.of(t, (int)(c / F));
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (w != 0.f) {
+        const long gi = shared ? 2 * EF + (c - EF) : c, ui = shared ? 2 * EF + FS + (c - EF) : EF + c;
+        float g[8], u[8];
+        Vec8<T>::load(gate_up + t * ld + gi, g);
+        Vec8<T>::load(gate_up + t * ld + ui, u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = moe_pair(w, g[e], u[e], limit, slope);
+    }
+    Vec8<T>::store(act + t * (EF + FS) + c, v);
+}
+
 extern "C" int mv_moe_swiglu_scale(const void* gate_up, long ld, const float* dense, int ld_dense, int n, int E, int F, int FS,
-                                   void* act, float limit, float slope, int dtype, hipStream_t stream) {
-    MV_REQUIRE(n >= 0 && E > 0 && F > 0 && FS >= 0 && ld >= 2L * E * F + 2L * FS && ld_dense >= E,
-               "moe_swiglu_scale: bad sizes n=%d E=%d F=%d shared=%d", n, E, F, FS);
-    MV_REQUIRE(gate_up && dense && act, "moe_swiglu_scale: missing operand");
+                                   void* act, float limit, float slope, const int* tokens, const int* table, int table_rows,
+                                   int top, int dtype, hipStream_t stream) {
+    MV_REQUIRE(n >= 0 && E > 0 && F > 0 && FS >= 0 && ld >= 2L * E * F + 2L * FS, "moe_swiglu_scale: bad sizes n=%d E=%d F=%d shared=%d",
+               n, E, F, FS);
+    MV_REQUIRE(gate_up && act && (table ? (tokens && table_rows > 0 && top > 0) : (dense && ld_dense >= E)),
+               "moe_swiglu_scale: missing operand");
     const long total = (long)n * ((long)E * F + FS);
     if (total == 0) return 0;
+    MoeWeights mw{dense, ld_dense, tokens, table, table_rows, top};
+    const size_t esz = mv_dtype_size(dtype);
+    if (F % 8 == 0 && FS % 8 == 0 && (ld * esz) % 16 == 0 && ((uintptr_t)gate_up % 16) == 0 && ((uintptr_t)act % 16) == 0) {
+        const long total8 = total / 8;
+        MV_DISPATCH_T(dtype, "moe_swiglu_scale",
+                      hipLaunchKernelGGL(moe_swiglu_scale_vec_kernel<T>, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, stream,
+                                         (const T*)gate_up, ld, mw, E, F, FS, (T*)act, total8, limit, slope));
+        return mv_check_launch("moe_swiglu_scale");
+    }
     MV_DISPATCH_T(dtype, "moe_swiglu_scale",
                   hipLaunchKernelGGL(moe_swiglu_scale_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
-                                     (const T*)gate_up, ld, dense, ld_dense, E, F, FS, (T*)act, total, limit, slope));
+                                     (const T*)gate_up, ld, mw, E, F, FS, (T*)act, total, limit, slope));
     return mv_check_launch("moe_swiglu_scale");
 }
 

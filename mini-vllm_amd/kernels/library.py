@@ -228,8 +228,9 @@ _OPTIONAL_SIGNATURES = {
     "mv_moe_route": (c_int, [c_void_p, c_long, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p,
                              c_void_p, c_void_p, c_void_p]),
     # gate_up, ld, dense, ld_dense, n, E, F, act, limit, slope, dtype, stream
+    # gate_up, ld, dense, ld_dense, n, E, F, FS, act, limit, slope, tokens, table, table_rows, top, dtype, stream
     "mv_moe_swiglu_scale": (c_int, [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_float, c_float,
-                                    c_int, c_void_p]),
+                                    c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     # y, ldy, h, ldh, dense, ld_dense, first, count, n, width, set, dtype, stream
     "mv_moe_identity_add": (c_int, [c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                     c_int, c_void_p]),

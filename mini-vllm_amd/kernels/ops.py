@@ -1053,24 +1053,38 @@ class Ops:
                       _weight_code(correction, "router correction") if correction is not None else DTYPE_F32, groups, keep,
                       top, float(sum_eps), flags, dense.data_ptr(), ids.data_ptr(), weights.data_ptr(), self._stream())
 
-    def moe_swiglu_scale(self, gate_up: torch.Tensor, dense: torch.Tensor, experts: int, ff: int, out: torch.Tensor,
-                         limit: float = 0.0, slope: float = 1.0, shared: int = 0) -> None:
+    def moe_swiglu_scale(self, gate_up: torch.Tensor, dense: Optional[torch.Tensor], experts: int, ff: int, out: torch.Tensor,
+                         limit: float = 0.0, slope: float = 1.0, shared: int = 0, table=None) -> None:
         """out[t, e, c] = dense[t, e] * silu(gate_up[t, e*ff + c]) * gate_up[t, experts*ff + e*ff + c] (zero where the
         weight is zero, whatever the products hold). With ``limit`` > 0 the clamped pair instead: g = min(gate, limit),
         u = clamp(up, -limit, limit), out = dense * g * sigmoid(slope * g) * (u + 1). With ``shared`` > 0 the rows hold
         that many gate and as many up columns of a shared expert behind the others', and out gets its pair, with the
-        weight one, behind the experts' columns."""
-        self._act(gate_up, "gate_up"); self._act(out, "expert activations"); _dev(dense, "dense weights")
+        weight one, behind the experts' columns. ``table`` = (token ids int32 [>= n], int32 [rows, top]) instead of
+        ``dense``: row t's experts are table[token_ids[t]], each with the weight 1 / top (what ``moe_table_route`` would
+        leave in ``dense``, looked up here instead)."""
+        self._act(gate_up, "gate_up"); self._act(out, "expert activations")
         n = gate_up.shape[0]
         if tuple(gate_up.shape) != (n, 2 * experts * ff + 2 * shared) or gate_up.stride(1) != 1 \
-                or tuple(out.shape) != (n, experts * ff + shared) \
-                or not out.is_contiguous() or dense.dtype != torch.float32 or dense.shape[0] != n or dense.shape[1] < experts \
-                or dense.stride(1) != 1:
+                or tuple(out.shape) != (n, experts * ff + shared) or not out.is_contiguous():
             raise KernelLibraryError("moe_swiglu_scale: operands do not fit")
+        tokens = rows = None
+        if table is not None:
+            tokens, rows = table
+            for t, name in ((tokens, "token ids"), (rows, "expert table")):
+                _dev(t, name)
+                if t.dtype != torch.int32 or not t.is_contiguous():
+                    raise KernelLibraryError(f"moe_swiglu_scale: {name} must be contiguous int32")
+            if tokens.numel() < n or rows.dim() != 2:
+                raise KernelLibraryError("moe_swiglu_scale: a token id for every row and a table [rows, top] are needed")
+        else:
+            _dev(dense, "dense weights")
+            if dense.dtype != torch.float32 or dense.shape[0] != n or dense.shape[1] < experts or dense.stride(1) != 1:
+                raise KernelLibraryError("moe_swiglu_scale: operands do not fit")
         self._note("mv_moe_swiglu_scale", self._size(gate_up, out), 8 * out.numel())
-        self.lib.call("mv_moe_swiglu_scale", gate_up.data_ptr(), gate_up.stride(0) if n > 1 else gate_up.shape[1], dense.data_ptr(),
-                      dense.stride(0) if n > 1 else dense.shape[1], n, experts, ff, int(shared), out.data_ptr(), float(limit),
-                      float(slope), self.code, self._stream())
+        self.lib.call("mv_moe_swiglu_scale", gate_up.data_ptr(), gate_up.stride(0) if n > 1 else gate_up.shape[1], _ptr(dense),
+                      (dense.stride(0) if n > 1 else dense.shape[1]) if dense is not None else 0, n, experts, ff, int(shared),
+                      out.data_ptr(), float(limit), float(slope), _ptr(tokens), _ptr(rows),
+                      rows.shape[0] if rows is not None else 0, rows.shape[1] if rows is not None else 0, self.code, self._stream())
 
     def moe_table_route(self, token_ids: torch.Tensor, table: torch.Tensor, experts: int, dense: torch.Tensor, ids: torch.Tensor,
                         weights: torch.Tensor) -> None:

@@ -32,6 +32,9 @@ VALUE_MIX_KEY = "values.first"     # where the first value-sharing layer leaves 
 
 
 def furanex_plan(config: FuranexConfig) -> ModelPlan:
+    # (sizes that config.json left out and no loader has filled in from the stored tensors take their defaults here,
+    # or are an error when they have none)
+    config = config.completed()
     hid = config.hidden_size
     norm = RMSNormSpec(size=hid, eps=config.norm_eps)
     first_mix = config.first_mixing_layer()
@@ -102,6 +105,16 @@ def furanex_tensor_name(config: FuranexConfig, loc: TensorLocation) -> str:
     raise KeyError(loc)
 
 
+def furanex_complete(config: FuranexConfig, source) -> FuranexConfig:
+    """The configuration with what only the stored tensors state, where config.json leaves it out: vocabulary and width
+    are the embedding's shape, the streams the length of ``l0.hc1.in``, head counts and sizes the rows of the projections,
+    the ranks the lengths of the latent norms, the rotated channels what ``dkv`` has beyond the latent, an expert's width
+    the rows of ``e0.gate``, the experts their number, ``top`` the table's columns, a shared expert's width the rows of
+    ``shared.gate`` (none when there is no such tensor)."""
+    names = set(source.names())
+    return config.completed(lambda name: tuple(source.shape(name)) if name in names else None)
+
+
 def furanex_ignorable(config: FuranexConfig) -> FrozenSet[str]:
     # the first value-sharing layer stores a blend weight it never uses; a layer without a feed-forward may still
     # store the norm and the stream weights in front of it
@@ -119,4 +132,5 @@ FURANEX = register_architecture(Architecture(
     plan=furanex_plan,
     tensor_name=furanex_tensor_name,
     ignorable=furanex_ignorable,
+    complete=furanex_complete,
 ))

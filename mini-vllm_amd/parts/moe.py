@@ -187,26 +187,34 @@ class RoutedExperts(FeedForward):
         dense = ws.get("moe.dense", (n, E), torch.float32)
         ids = ws.get("moe.ids", (n, spec.top), torch.int32)
         weights = ws.get("moe.weights", (n, spec.top), torch.float32)
-        if spec.router == "table":
+        by_table = spec.router == "table"
+        grouped = bool(n_e) and ops.use_fast_kernels and self.wants_grouped(n)
+        if by_table and grouped:
             ops.moe_table_route(ctx.token_ids, self.table, n_e, dense, ids, weights)
+        elif by_table:
+            pass                  # all experts at once: the activation kernel looks the weights up itself
         else:
             logits = ws.get("moe.logits", (n, E), torch.float32)
             ops.gemm(x, self.w_router, logits)
             ops.moe_route(logits, self.correction, spec.groups, spec.keep_groups, spec.top, spec.weight_sum_eps, dense, ids, weights,
                           scoring=spec.scoring, group_worth=spec.group_worth, normalize=spec.normalize)
         y = ws.get("ffn.out", (n, spec.hidden_size), rt.dtype)
-        if n_e and ops.use_fast_kernels and self.wants_grouped(n) and self._grouped(x, ctx, dense, ids, weights, y):
+        if grouped and self._grouped(x, ctx, dense, ids, weights, y):
             if apart:
                 self._add_shared(x, y)
             return y
+        if grouped and by_table:
+            grouped = False       # the sizes were not served after all: the lists are there, the kernel below takes the table
         if n_e:
             gu = ws.get("moe.gate_up", (n, 2 * n_e * F + 2 * FS), rt.dtype)
             ops.gemm(x, self.w_gate_up, gu)
             act = ws.get("moe.act", (n, n_e * F + FS), rt.dtype)
+            table = (ctx.token_ids, self.table) if by_table else None
             if spec.activation == "clamped":
-                ops.moe_swiglu_scale(gu, dense, n_e, F, act, limit=spec.limit, slope=spec.gate_slope, shared=FS)
+                ops.moe_swiglu_scale(gu, None if by_table else dense, n_e, F, act, limit=spec.limit, slope=spec.gate_slope,
+                                     shared=FS, table=table)
             else:
-                ops.moe_swiglu_scale(gu, dense, n_e, F, act, shared=FS)
+                ops.moe_swiglu_scale(gu, None if by_table else dense, n_e, F, act, shared=FS, table=table)
             ops.gemm(act, self.w_down, y)
             if apart:
                 self._add_shared(x, y)

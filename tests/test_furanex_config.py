@@ -39,10 +39,41 @@ def test_defaults():
     m = raw["layers"][0]["mixer"]
     del m["kv_heads"], m["vdim"], m["scale"], m["v_mix"], m["rot"]["scaling"]
     raw["layers"][1]["mixer"]["v_mix"] = False
-    cfg = FuranexConfig.from_dict(raw)
+    cfg = FuranexConfig.from_dict(raw).completed()
     l0 = cfg.layers[0].mixer
     assert cfg.embedding_scale == 1.0 and cfg.streams == 0 and l0.kv_heads == l0.heads and l0.vdim == l0.dim
     assert l0.scale == l0.dim ** -0.5 and not l0.v_mix and l0.rot.stretch is None and cfg.first_mixing_layer() is None
+    assert cfg.layers[0].mlp.shared_ff == 0 and cfg.layers[1].mlp.shared_ff == 12
+
+
+@pytest.mark.parametrize("name", sorted(FUR))
+def test_sizes_left_out_are_read_from_the_stored_shapes(name):
+    """Everything a stored tensor's shape states may be left out of config.json: the completed configuration is the one
+    that states it all. What no shape states (a head's size when the head count is left out too) is an error."""
+    full = FuranexConfig.from_dict(FUR[name]).completed()
+    raw = copy.deepcopy(FUR[name])
+    for key in ("vocab", "width", "streams"):
+        raw.pop(key, None)
+    for layer in raw["layers"]:
+        m = layer["mixer"]
+        for key in ("heads", "kv_heads", "vdim", "q_rank", "kv_rank", "rot_dim"):
+            m.pop(key, None)
+        if layer["type"] == "latent_attention":
+            m.pop("dim")
+        if layer.get("mlp"):
+            layer["mlp"].pop("shared", None)
+            layer["mlp"]["expert"].pop("ff")
+            layer["mlp"]["router"] = {}
+    shapes = tensor_shapes(FUR[name])
+    thin = FuranexConfig.from_dict(raw)
+    assert thin.vocab_size == -1 and thin.layers[0].mixer.heads == -1
+    assert thin.completed(lambda n: shapes.get(n)) == full
+    with pytest.raises(ConfigError):
+        thin.completed()
+    attn = next(l for l in raw["layers"] if l["type"] == "attention")
+    del attn["mixer"]["dim"]
+    with pytest.raises(ConfigError):
+        FuranexConfig.from_dict(raw).completed(lambda n: shapes.get(n))
 
 
 def _broken(name, edit):
@@ -68,7 +99,7 @@ def _broken(name, edit):
 ])
 def test_configuration_errors(name, edit):
     with pytest.raises(ConfigError):
-        FuranexConfig.from_dict(_broken(name, edit))
+        FuranexConfig.from_dict(_broken(name, edit)).completed()
 
 
 def test_plan_and_memory():

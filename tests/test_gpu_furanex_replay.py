@@ -295,3 +295,24 @@ def test_configurations_drawn_at_random(tmp_path, seed, fast_sizes):
         else:
             tol = bf16_tolerance(max(rel_err(plain_logits_bf16(cfg, weights, reqs[rid])[p], want[rid][p]) for rid, p in sample))
         judge([rel_err(row, want[rid][pos]) for (rid, pos), row in got.items()], tol, dtype, f"random configuration {seed}")
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_sizes_left_out_of_the_configuration(cases, tmp_path, name):
+    """A folder whose config.json leaves out everything the stored tensors' shapes state serves like the full one."""
+    import copy
+    case = cases[(name, "mild")]
+    raw = copy.deepcopy(case.cfg)
+    for key in ("vocab", "width", "streams"):
+        raw.pop(key, None)
+    for layer in raw["layers"]:
+        for key in ("heads", "kv_heads", "vdim", "q_rank", "kv_rank", "rot_dim"):
+            layer["mixer"].pop(key, None)
+        if layer["type"] == "latent_attention":
+            layer["mixer"].pop("dim")
+        if layer.get("mlp"):
+            layer["mlp"] = {"kind": "moe"}
+    thin = type("Thin", (), {"dir": write_model_dir(str(tmp_path / "thin"), raw, case.weights), "page": case.page})()
+    steps = trace_tools.portions(case.reqs)
+    got = trace_tools.collect(steps, runner_for(thin, "float32", steps).run_step)
+    assert len(got) == case.check(got, "float32", f"{name} with sizes left out")
