@@ -245,10 +245,10 @@ extern "C" int mv_hyper_step(float* lanes, long plane, const float* first, int S
     MV_REQUIRE(y || first || w_in || total, "hyper_step: nothing to do");
     if (n == 0) return 0;
     WeightPtr wn{w_norm, norm_dtype};
-    const size_t esz = mv_dtype_size(dtype);
+    // four columns at a time: rows of floats 16 bytes, rows of the activation type at least 8 bytes aligned
     const bool aligned = W % 4 == 0 && plane % 4 == 0 && ((uintptr_t)lanes % 16) == 0 && ((uintptr_t)first % 16) == 0 &&
-                         ((uintptr_t)total % 16) == 0 && ((uintptr_t)y % 16) == 0 && (ldy * esz) % (4 * esz) == 0 &&
-                         ((uintptr_t)h % 16) == 0 && ldh % 4 == 0 && ldy % 4 == 0 && ((uintptr_t)w_norm % 16) == 0;
+                         ((uintptr_t)total % 16) == 0 && ((uintptr_t)y % 16) == 0 && ldy % 4 == 0 &&
+                         ((uintptr_t)h % 16) == 0 && ldh % 4 == 0 && ((uintptr_t)w_norm % 16) == 0;
     if (aligned && S <= 4 && W <= 4 * HY_THREADS * 8) {
         bool took = false;
 #define HY_S(SS)                                                                                                                \

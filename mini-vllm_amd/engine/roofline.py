@@ -68,7 +68,7 @@ KERNELS_OF: Dict[str, Tuple[str, Optional[str], int]] = {
     "mv_attention_latent_mfma": (r"\battention_latent_mfma_kernel", None, 1),
     "mv_attention_latent_split": (r"\battention_latent_split_kernel", r"\battention_latent_join_kernel", 2),
     "mv_moe_route": (r"\bmoe_route_kernel", None, 1),
-    "mv_moe_swiglu_scale": (r"\bmoe_swiglu_scale_kernel", None, 1),
+    "mv_moe_swiglu_scale": (r"\bmoe_swiglu_scale(_vec)?_kernel", None, 1),
     "mv_moe_identity_add": (r"\bmoe_identity_add_kernel", None, 1),
     "mv_scale_f32": (r"\bscale_f32_kernel", None, 1),
     "mv_input_conv": (r"\binput_conv(_vec)?_kernel", r"\bconv_state_kernel", 2),

@@ -7,6 +7,8 @@ from __future__ import annotations
 
 from typing import Optional
 
+import os
+
 import torch
 
 from . import library
@@ -79,6 +81,12 @@ TILE_BIG_MIN_M = 9
 TILE_BIG_MAX_M = 256
 TILE_HUGE_WEIGHT = 96 * 1024 * 1024           # bytes
 TILE_HUGE_MIN_M = 8
+# weights with long rows (the down matrices of a mixture's experts side by side: K = experts x width): the
+# weight-streaming product splits such a K over few waves and reaches 2.2 TB/s on them, the tiled one splits it over
+# workgroups. Measured with MV_TILE_LONG_ROWS=0 and 1, decode at batch 8 of the 0.6B-sized mixtures (K = 25,344, N = 1,024):
+# Furanex 3.375 -> 3.323 ms a step, Dutilix 2.467 -> 2.446, Zedudra 2.321 -> 2.294; batch 1 unchanged
+TILE_LONG_ROWS_K = 16384
+TILE_LONG_ROWS_RATIO = 8                      # K >= ratio * N
 # most rows for which residual add and norm are fused into the following product
 FUSED_NORM_MAX_M = 16
 # the fused kernel keeps the rows in registers: at most 8 waves x 4 chunks of 512 columns
@@ -1655,6 +1663,8 @@ class Ops:
         if weight_bytes >= TILE_BIG_WEIGHT:
             if M < TILE_BIG_MIN_M:
                 if N * K >= MID_ALWAYS_WEIGHT:
+                    return True
+                if K >= TILE_LONG_ROWS_K and K >= TILE_LONG_ROWS_RATIO * N and os.environ.get("MV_TILE_LONG_ROWS", "1") != "0":
                     return True
                 return M >= TILE_HUGE_MIN_M and weight_bytes >= TILE_HUGE_WEIGHT and not fold_offered
             return M <= TILE_BIG_MAX_M

@@ -30,6 +30,12 @@ output by sigmoid(z) on its own; ``group_worth`` "top2" ranks a group by the sum
 instead of its largest; ``normalize`` False uses the chosen scores themselves as weights; ``activation``
 "clamped" replaces the gated SiLU pair by g = min(gate, limit), u = clamp(up, -limit, limit),
 g * sigmoid(gate_slope * g) * (u + 1).
+
+``router`` "table": there is no router. A stored integer table [``table_rows``, ``top``] names the experts of every
+token id (the step's ``ctx.token_ids``), each with the weight 1 / top; with all experts at once the activation kernel
+looks the weights up itself, the chosen-pairs path gets the usual lists from ``moe_table_route``. ``shared_size`` > 0:
+a shared expert (a gated pair like the others) runs for every token and is added: its rows ride in the two packed
+products, or, where steps may take the chosen pairs only, it keeps two products of its own.
 """
 from __future__ import annotations
 
