@@ -189,9 +189,9 @@ def furanex_shape(name: str, layers: int = None, streams: int = 4, experts: int 
     q = QWEN3_SHAPES[name]
     n = layers or q["num_hidden_layers"]
     hid, hd = q["hidden_size"], q["head_dim"]
-    stretch = {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+    stretch = {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}
     attention = {"heads": q["num_attention_heads"], "kv_heads": q["num_key_value_heads"], "dim": hd, "vdim": hd,
-                 "scale": 0.125, "v_mix": True, "rot": {"dims": hd, "base": q["rope_theta"], "scaling": dict(stretch)}}
+                 "scale": 8.0 / hd, "v_mix": True, "rot": {"dims": hd, "base": q["rope_theta"], "scaling": dict(stretch)}}
     latent = {"heads": q["num_attention_heads"], "dim": hd, "rot_dim": 64, "vdim": hd, "q_rank": max(64, hid // 4),
               "kv_rank": 256, "scale": (hd + 64) ** -0.5, "rot": {"dims": 64, "base": 10000.0, "scaling": dict(stretch)}}
     mlp = {"kind": "moe", "expert": {"ff": q["intermediate_size"] // top}, "router": {"experts": experts, "top": top}}

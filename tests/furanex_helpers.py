@@ -56,11 +56,11 @@ FUR_B = {"architecture": "Furanex", "vocab": 77, "width": 50, "streams": 2, "nor
                     attn(2, 1, 6, 4, 2, 30.0, 0.4, None, v_mix=False),
                     attn(6, 3, 12, 14, 6, 77.0, 0.3, moe(10, 4, 4, shared=26))]}
 # C: sizes that resemble a real model's heads (64 and 128, latents of 128 and 256 with 32 and 64 rotated channels),
-# four streams, as the MFMA kernels take them
+# four streams, as the MFMA and vector kernels take them
 FUR_C = {"architecture": "Furanex", "vocab": 512, "width": 256, "streams": 4, "norm": {"eps": 1e-6}, "embedding": {"scale": 16.0},
-         "layers": [attn(8, 2, 64, 64, 64, 1000000.0, 0.125, moe(64, 12, 1, shared=96), scaling=stretch(4.0, 1024, 32.0, 1.0)),
-                    latent(4, 32, 32, 48, 128, 128, 10000.0, 0.125, moe(64, 12, 1, shared=96), scaling=stretch(2.0, 512, 32.0, 1.0)),
-                    attn(8, 2, 64, 64, 64, 1000000.0, 0.125, moe(128, 8, 2, shared=64), scaling=stretch(4.0, 1024, 32.0, 1.0)),
+         "layers": [attn(6, 2, 64, 64, 64, 500000.0, 0.1, moe(96, 10, 2, shared=64), scaling=stretch(8.0, 2048, 16.0, 2.0)),
+                    latent(8, 64, 32, 32, 96, 128, 20000.0, 0.1, moe(96, 10, 2, shared=64), scaling=stretch(4.0, 256, 16.0, 1.0)),
+                    attn(6, 2, 64, 64, 64, 500000.0, 0.1, moe(128, 8, 1, shared=32), scaling=stretch(8.0, 2048, 16.0, 2.0)),
                     latent(16, 64, 64, 64, 96, 256, 50000.0, 0.09, moe(32, 4, 2)),
                     attn(2, 1, 128, 128, 128, 10000.0, 0.09, None, v_mix=False)]}
 # D: one stream, one head everywhere, no rotation at all in one layer and no rotated part in the latent layer, every

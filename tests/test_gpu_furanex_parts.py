@@ -66,7 +66,7 @@ class Paged:
 # residual streams
 # ---------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("S, W", [(4, 320), (3, 48), (2, 50), (1, 32), (5, 64), (8, 40), (4, 1024), (2, 4096), (3, 8200), (4, 8192)])
+@pytest.mark.parametrize("S, W", [(4, 384), (3, 48), (2, 50), (1, 32), (5, 64), (8, 40), (4, 1024), (2, 4096), (3, 8200), (4, 8192)])
 def test_stream_step(dtype, S, W):
     """The three shapes of the step against the plain read and write: widths and stream counts the vector kernel takes
     (a multiple of four columns up to 8,192, at most four streams) and those it leaves to the general one."""
@@ -142,7 +142,7 @@ def build_attention(rt, m, w, width, eps, mixes):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H, G, D, Dv, rot, width, page, mixes", [
-    (4, 2, 16, 8, 12, 48, 16, True), (3, 3, 10, 14, 10, 50, 8, False), (8, 2, 64, 64, 64, 128, 16, True),
+    (4, 2, 16, 8, 12, 48, 16, True), (3, 3, 10, 14, 10, 50, 8, False), (6, 3, 64, 64, 64, 128, 16, True),
     (2, 1, 128, 128, 128, 64, 16, True), (2, 2, 8, 20, 4, 32, 4, True), (1, 1, 12, 12, 0, 40, 16, False),
     (4, 1, 64, 64, 32, 96, 16, True), (6, 2, 64, 32, 64, 64, 16, False)])
 def test_attention_whole_in_portions_and_token_by_token(dtype, H, G, D, Dv, rot, width, page, mixes):
@@ -220,7 +220,7 @@ def test_one_key_that_stands_out_is_found_wherever_it_lies(dtype, single, D, Dv)
 # ---------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H, D, Dr, Dv, Q, R, width, page", [(3, 12, 4, 8, 24, 16, 48, 16), (5, 6, 2, 10, 14, 18, 50, 8),
-                                                             (4, 32, 32, 48, 128, 128, 320, 16), (1, 20, 0, 6, 10, 12, 32, 4),
+                                                             (6, 24, 32, 40, 64, 128, 192, 16), (1, 20, 0, 6, 10, 12, 32, 4),
                                                              (16, 64, 64, 64, 96, 256, 128, 16), (2, 16, 16, 8, 32, 64, 64, 16)])
 def test_latent_attention_whole_in_portions_and_token_by_token(dtype, H, D, Dr, Dv, Q, R, width, page):
     from minivllm_amd.parts.latent_attention import LatentAttention, LatentAttentionSpec
@@ -292,7 +292,7 @@ def build_mixture(rt, w, hid, F, E, top, FS, vocab, **options):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hid, F, E, top, FS", [(48, 24, 5, 2, 40), (50, 22, 3, 1, 0), (320, 64, 12, 1, 96), (40, 10, 4, 4, 26), (64, 16, 1, 1, 8)])
+@pytest.mark.parametrize("hid, F, E, top, FS", [(48, 24, 5, 2, 40), (50, 22, 3, 1, 0), (256, 64, 10, 1, 128), (40, 10, 4, 4, 26), (64, 16, 1, 1, 8)])
 def test_table_mixture_against_the_plain_one(dtype, hid, F, E, top, FS):
     """A row's experts follow its token id alone: the same ids in another order, beside other rows, give the same rows."""
     vocab, n = 37, 60
