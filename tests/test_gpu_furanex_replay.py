@@ -19,6 +19,10 @@ LENGTHS = {"A": [70, 5, 45, 21, 33, 2], "B": [88, 40, 66, 3, 58], "C": [150, 17,
            "E": [40, 3, 65, 129]}
 PAGE = {"A": 16, "B": 8, "C": 16, "D": 16, "E": 8}
 GAINS = {"sharp": 12.0, "mild": 1.0}
+# q and k are unit vectors, so a score is at most scale x dim: the heads of 64 and 128 channels of C get a smaller factor
+# (their largest score is then 26 instead of 77, beyond which bfloat16 rounding of the cached keys alone moves the logits
+# by a tenth)
+SHARP_OF = {"C": 4.0}
 
 
 def judge(errors, tol, dtype, what):
@@ -32,7 +36,7 @@ def judge(errors, tol, dtype, what):
 class Case:
     def __init__(self, name, tmp, kind):
         self.name, self.kind, self.page = name, kind, PAGE[name]
-        self.cfg = sharpened(FUR[name], GAINS[kind])
+        self.cfg = sharpened(FUR[name], SHARP_OF.get(name, GAINS[kind]) if kind == "sharp" else GAINS[kind])
         self.weights = make_weights(self.cfg, seed=sum(map(ord, name)) + 1, key_gain=2.0 if kind == "sharp" else 1.0)
         self.dir = write_model_dir(str(tmp / f"fur{name}_{kind}"), self.cfg, self.weights)
         self.reqs = {f"r{i}": random_tokens(self.cfg, n, seed=100 + i) for i, n in enumerate(LENGTHS[name])}
