@@ -144,7 +144,7 @@ def build_attention(rt, m, w, width, eps, mixes):
 @pytest.mark.parametrize("H, G, D, Dv, rot, width, page, mixes", [
     (4, 2, 16, 8, 12, 48, 16, True), (3, 3, 10, 14, 10, 50, 8, False), (6, 3, 64, 64, 64, 128, 16, True),
     (2, 1, 128, 128, 128, 64, 16, True), (2, 2, 8, 20, 4, 32, 4, True), (1, 1, 12, 12, 0, 40, 16, False),
-    (4, 1, 64, 64, 32, 96, 16, True), (6, 2, 64, 32, 64, 64, 16, False)])
+    (4, 1, 64, 64, 32, 96, 16, True), (6, 2, 64, 32, 64, 64, 16, False), (2, 2, 256, 256, 256, 64, 16, True)])
 def test_attention_whole_in_portions_and_token_by_token(dtype, H, G, D, Dv, rot, width, page, mixes):
     n, eps = 150, 1e-5
     m, w, h, first_values = attention_case(H, G, D, Dv, rot, width, seed=H * D + Dv, n=n, mixes=mixes)
@@ -347,3 +347,23 @@ def test_chosen_pairs_only_against_all_experts(n, hid, F, E, top, FS):
     want = plain.table_mixture(x.double(), ids, {k: (v.double() if v.is_floating_point() else v) for k, v in w.items()}, "m.", f)
     close(outs[True], want, 2e-2, "chosen pairs only against the plain mixture")
     close(outs[True], outs[False].double(), 2e-2, "chosen pairs only against all experts")
+
+
+@pytest.mark.parametrize("M", [1, 3, 8])
+@pytest.mark.parametrize("N, K", [(1024, 16384), (512, 20480), (1024, 25344)])
+def test_products_against_weights_with_long_rows(M, N, K):
+    """The down matrices of a mixture's experts side by side are a weight with very long rows; steps of few rows send it
+    to the tiled product, whose workgroups split the row."""
+    ops = ops_for(torch.bfloat16)
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(N, K, generator=g) / K ** 0.5).to(torch.bfloat16).to(DEV)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.ledger = []
+    done = ops.gemm(a, w, out)
+    if done is not None and not isinstance(done, torch.Tensor):
+        done.materialize()
+    torch.cuda.synchronize()
+    assert [e[0] for e in ops.ledger][:1] == ["mv_gemm_tile"], [e[0] for e in ops.ledger]
+    ops.ledger = None
+    close(out, a.double() @ w.double().T, 1e-2, "long rows")
