@@ -83,8 +83,8 @@ TILE_HUGE_WEIGHT = 96 * 1024 * 1024           # bytes
 TILE_HUGE_MIN_M = 8
 # weights with long rows (the down matrices of a mixture's experts side by side: K = experts x width): the
 # weight-streaming product splits such a K over few waves and reaches 2.2 TB/s on them, the tiled one splits it over
-# workgroups. Measured with MV_TILE_LONG_ROWS=0 and 1, decode at batch 8 of the 0.6B-sized mixtures (K = 25,344, N = 1,024):
-# Furanex 3.375 -> 3.323 ms a step, Dutilix 2.467 -> 2.446, Zedudra 2.321 -> 2.294; batch 1 unchanged
+# workgroups, sixteen ways for such rows (``tile_plan``). Measured with MV_TILE_LONG_ROWS=0 and 1, decode at batch 8 of the
+# 0.6B-sized mixtures (K = 25,344, N = 1,024): Furanex 3.375 -> 3.22 ms a step (3.32 with eight splits), Dutilix 2.467 -> 2.40
 TILE_LONG_ROWS_K = 16384
 TILE_LONG_ROWS_RATIO = 8                      # K >= ratio * N
 # most rows for which residual add and norm are fused into the following product
