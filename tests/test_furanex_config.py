@@ -122,8 +122,8 @@ def test_plan_and_memory():
     assert all(l.block.kind == "pre_norm" for l in arch.plan(cfg).layers)
 
 
-@pytest.mark.parametrize("dims, base, stretch", [(12, 5000.0, (3.0, 64, 16.0, 2.0)), (64, 1e6, (4.0, 1024, 32.0, 1.0)),
-                                                 (32, 1e4, (2.0, 512, 32.0, 1.0)), (8, 200.0, (2.0, 4000, 1000.0, 0.001)),
+@pytest.mark.parametrize("dims, base, stretch", [(12, 5000.0, (3.0, 64, 16.0, 2.0)), (64, 5e5, (8.0, 2048, 16.0, 2.0)),
+                                                 (48, 2e4, (4.0, 256, 16.0, 1.0)), (8, 200.0, (2.0, 4000, 1000.0, 0.001)),
                                                  (4, 300.0, (8.0, 16, 4.0, 0.5)), (128, 1e6, (40.0, 4096, 32.0, 1.0))])
 def test_stretched_frequencies(dims, base, stretch):
     from minivllm_amd.parts.rope import stretched_frequencies
